@@ -48,6 +48,9 @@ def _flags():
         "-Wno-unused-variable",
         "-ffp-contract=fast",
         "-munsafe-fp-atomics",
+        # no packed-fp32 VALU forms: the compiler forms them from ordinary float code, and some of them have
+        # returned wrong values on this hardware
+        "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     ]
 
 

@@ -72,6 +72,31 @@ void launch_quant_fp8_rows(const void* w, void* q, void* scale, int64_t N, int64
 void launch_quant_fp8_rows_ld(const void* x, int64_t ldx, void* q, void* scale, int64_t M, int64_t K, hipStream_t st);
 void launch_dequant_fp8_rows(const void* q, const void* scale, void* w, int64_t N, int64_t K, hipStream_t st);
 
+// fp32 residual stream, strided / grouped GEMMs in either storage type, latent attention, mixture of experts
+void launch_embed_scaled(const void* ids, const void* table, void* x, int T_, int H, int vocab, float scale, int dt,
+                         hipStream_t st);
+void launch_resid_add_norm(void* x, const void* a, int64_t lda, const void* b, int64_t ldb, const void* w, float woff,
+                           float eps, void* y, int64_t ldy, int T_, int H, int dt, hipStream_t st);
+void launch_gemm_any(const void* A, const void* B, void* C, int M, int N, int K, int batch, int64_t sAb, int64_t sAm,
+                     int64_t sBb, int64_t sBn, int64_t sBk, int64_t sCb, int64_t sCm, int da, int db, int dc,
+                     hipStream_t st);
+void launch_latent_norm_cache(const void* src, int64_t ld, int off, const void* w, float eps, void* cache,
+                              const void* slots, int T_, int R, int dt, hipStream_t st);
+void launch_latent_attn(const void* qa, int64_t ldq, const void* cache, const void* bt, int maxb, const void* cu_q,
+                        const void* ctx_lens, void* out, int64_t ldo, int T_, int B, int H, int R, int bs, int window,
+                        float scale, int dt, hipStream_t st);
+void launch_moe_route(const void* z, const void* corr, void* idx, void* wts, int T_, int E, int top, hipStream_t st);
+void launch_moe_group(const void* idx, int P, int E, int maxt, void* meta, void* order, void* place, hipStream_t st);
+void launch_moe_gate_up(const void* h, int64_t ldh, const void* wg, const void* wu, const void* meta,
+                        const void* order, void* act, int E, int maxt, int top, int F, int K, float limit,
+                        float alpha, int dt, hipStream_t st);
+void launch_moe_down(const void* act, const void* wd, const void* meta, void* y, int E, int maxt, int N, int F,
+                     int dt, hipStream_t st);
+void launch_moe_combine(const void* y, const void* place, const void* wts, const void* shared_, int64_t lds_,
+                        void* out, int T_, int N, int top, int dt, hipStream_t st);
+void launch_glu_clamp(const void* gu, int64_t ldg, void* out, int64_t ldo, int T_, int F, float limit, float alpha,
+                      int dt, hipStream_t st);
+
 void register_runtime(py::module_& m);  // host-side C++ runtime (runtime.cpp)
 void register_comm(py::module_& m);     // RCCL communicator (comm.cpp)
 void register_ctrl(py::module_& m);     // shared-memory control ring (ctrl.cpp)
@@ -207,6 +232,45 @@ PYBIND11_MODULE(_C, m) {
   m.def("dequant_fp8_rows", [](uintptr_t q, uintptr_t scale, uintptr_t w, int64_t N, int64_t K, uintptr_t st) {
     launch_dequant_fp8_rows(CP(q), CP(scale), P(w), N, K, S(st));
   });
+  m.def("embed_scaled", [](uintptr_t ids, uintptr_t table, uintptr_t x, int T, int H, int V, float scale, int dt,
+                           uintptr_t st) { launch_embed_scaled(CP(ids), CP(table), P(x), T, H, V, scale, dt, S(st)); });
+  m.def("resid_add_norm", [](uintptr_t x, uintptr_t a, int64_t lda, uintptr_t b, int64_t ldb, uintptr_t w, float woff,
+                             float eps, uintptr_t y, int64_t ldy, int T, int H, int dt, uintptr_t st) {
+    launch_resid_add_norm(P(x), CP(a), lda, CP(b), ldb, CP(w), woff, eps, P(y), ldy, T, H, dt, S(st));
+  });
+  m.def("gemm_any", [](uintptr_t A, uintptr_t B, uintptr_t C, int M, int N, int K, int batch, int64_t sAb, int64_t sAm,
+                       int64_t sBb, int64_t sBn, int64_t sBk, int64_t sCb, int64_t sCm, int da, int db, int dc,
+                       uintptr_t st) {
+    launch_gemm_any(CP(A), CP(B), P(C), M, N, K, batch, sAb, sAm, sBb, sBn, sBk, sCb, sCm, da, db, dc, S(st));
+  });
+  m.def("latent_norm_cache", [](uintptr_t src, int64_t ld, int off, uintptr_t w, float eps, uintptr_t cache,
+                                uintptr_t slots, int T, int R, int dt, uintptr_t st) {
+    launch_latent_norm_cache(CP(src), ld, off, CP(w), eps, P(cache), CP(slots), T, R, dt, S(st));
+  });
+  m.def("latent_attn", [](uintptr_t qa, int64_t ldq, uintptr_t cache, uintptr_t bt, int maxb, uintptr_t cu,
+                          uintptr_t ctx, uintptr_t out, int64_t ldo, int T, int B, int H, int R, int bs, int window,
+                          float scale, int dt, uintptr_t st) {
+    launch_latent_attn(CP(qa), ldq, CP(cache), CP(bt), maxb, CP(cu), CP(ctx), P(out), ldo, T, B, H, R, bs, window,
+                       scale, dt, S(st));
+  });
+  m.def("moe_route", [](uintptr_t z, uintptr_t corr, uintptr_t idx, uintptr_t wts, int T, int E, int top,
+                        uintptr_t st) { launch_moe_route(CP(z), CP(corr), P(idx), P(wts), T, E, top, S(st)); });
+  m.def("moe_group", [](uintptr_t idx, int Pn, int E, int maxt, uintptr_t meta, uintptr_t order, uintptr_t place,
+                        uintptr_t st) { launch_moe_group(CP(idx), Pn, E, maxt, P(meta), P(order), P(place), S(st)); });
+  m.def("moe_gate_up", [](uintptr_t h, int64_t ldh, uintptr_t wg, uintptr_t wu, uintptr_t meta, uintptr_t order,
+                          uintptr_t act, int E, int maxt, int top, int F, int K, float limit, float alpha, int dt,
+                          uintptr_t st) {
+    launch_moe_gate_up(CP(h), ldh, CP(wg), CP(wu), CP(meta), CP(order), P(act), E, maxt, top, F, K, limit, alpha, dt,
+                       S(st));
+  });
+  m.def("moe_down", [](uintptr_t act, uintptr_t wd, uintptr_t meta, uintptr_t y, int E, int maxt, int N, int F, int dt,
+                       uintptr_t st) { launch_moe_down(CP(act), CP(wd), CP(meta), P(y), E, maxt, N, F, dt, S(st)); });
+  m.def("moe_combine", [](uintptr_t y, uintptr_t place, uintptr_t wts, uintptr_t sh, int64_t lds_, uintptr_t out, int T,
+                          int N, int top, int dt, uintptr_t st) {
+    launch_moe_combine(CP(y), CP(place), CP(wts), CP(sh), lds_, P(out), T, N, top, dt, S(st));
+  });
+  m.def("glu_clamp", [](uintptr_t gu, int64_t ldg, uintptr_t out, int64_t ldo, int T, int F, float limit, float alpha,
+                        int dt, uintptr_t st) { launch_glu_clamp(CP(gu), ldg, P(out), ldo, T, F, limit, alpha, dt, S(st)); });
   register_runtime(m);
   register_comm(m);
   register_ctrl(m);

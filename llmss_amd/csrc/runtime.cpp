@@ -184,6 +184,60 @@ class Scheduler {
     seqs_.erase(it);
   }
 
+  // A step dictated from outside (replaying a recorded schedule; tests of cache reuse): sequence ids[i] is fed
+  // counts[i] further tokens in this step, whatever budget or chunking schedule() would have chosen. An unknown
+  // id is admitted as a running sequence without tokens; a known one grows. The same allocator, slot mapping and
+  // block tables as schedule() serve it, and finish(id) gives the blocks back. Rows come out as a step needs
+  // them: single tokens after a cached prefix first (num_decode), then the portions; `ids` holds that order.
+  // All-or-nothing: when the pool cannot hold the whole step, nothing is changed and an exception is raised.
+  StepBatch feed(const std::vector<int64_t>& ids, const std::vector<int>& counts) {
+    if (ids.size() != counts.size()) throw std::invalid_argument("Scheduler.feed: length mismatch");
+    int need = 0, fresh = 0;
+    for (size_t i = 0; i < ids.size(); ++i) {
+      if (counts[i] <= 0) throw std::invalid_argument("Scheduler.feed: a sequence needs at least one token");
+      for (size_t j = 0; j < i; ++j)
+        if (ids[j] == ids[i]) throw std::invalid_argument("Scheduler.feed: duplicate id in one step");
+      auto it = seqs_.find(ids[i]);
+      int have_tok = 0, have_blk = 0;
+      if (it == seqs_.end()) {
+        ++fresh;
+      } else {
+        const auto& s = it->second;
+        if (s.status != 1 || s.num_computed != s.num_tokens)
+          throw std::runtime_error("Scheduler.feed: sequence is queued or has tokens not yet computed");
+        have_tok = s.num_tokens;
+        have_blk = (int)s.blocks.size();
+      }
+      if (have_tok + counts[i] > max_len_) throw std::invalid_argument("Scheduler.feed: sequence exceeds max_model_len");
+      need += std::max(0, blocks_for(have_tok + counts[i]) - have_blk);
+    }
+    if ((int)running_.size() + fresh > max_seqs_) throw std::runtime_error("Scheduler.feed: no free sequence slot");
+    if (!alloc_.can_allocate(need)) throw std::runtime_error("Scheduler.feed: KV pool exhausted");
+    StepBatch b;
+    for (int pass = 0; pass < 2; ++pass) {  // pass 0: single tokens after a prefix, pass 1: portions
+      for (size_t i = 0; i < ids.size(); ++i) {
+        auto it = seqs_.find(ids[i]);
+        const bool emitted = std::find(b.ids.begin(), b.ids.end(), ids[i]) != b.ids.end();
+        const bool dec = counts[i] == 1 && it != seqs_.end() && it->second.num_tokens > 0;
+        if (emitted || (pass == 0 && !dec)) continue;
+        if (it == seqs_.end()) {
+          SeqState s{ids[i], 0, max_len_, 0, 0, {}, 1, counter_++};
+          it = seqs_.emplace(ids[i], s).first;
+          running_.push_back(ids[i]);
+        }
+        auto& s = it->second;
+        s.num_tokens += counts[i];
+        s.prompt_len = s.num_tokens;
+        grow(s, s.num_tokens);
+        emit(b, s, counts[i]);
+      }
+      if (pass == 0) b.num_decode = (int)b.ids.size();
+    }
+    b.kind = (b.num_decode == (int)b.ids.size()) ? 2 : 1;
+    fill_tables(b);
+    return b;
+  }
+
   void abort(int64_t id) { finish(id); }
 
   // One step. When prompt chunks hold the pool and none of them can grow while nothing decodes (the
@@ -721,6 +775,7 @@ void register_runtime(py::module_& m) {
       .def("finish", &Scheduler::finish)
       .def("abort", &Scheduler::abort)
       .def("schedule", &Scheduler::schedule)
+      .def("feed", &Scheduler::feed)
       .def("num_waiting", &Scheduler::num_waiting)
       .def("num_running", &Scheduler::num_running)
       .def("num_prefilling", &Scheduler::num_prefilling)

@@ -8,7 +8,9 @@ import torch
 
 from ..models.config import ModelConfig, get_preset
 from ..models.decoder import DecoderLM
-from ..models.weights import load_hf_weights, load_shard, random_weights, save_shard, shard_cache_path
+from ..models.layered import LayeredLM, create_model
+from ..models.weights import (load_hf_weights, load_shard, load_timisun_weights, random_timisun_weights,
+                              random_weights, save_shard, shard_cache_path)
 from ..parallel.dist import TPGroup
 from ..utils.checkpoint import CheckpointReader, weight_files
 from .engine import LLMEngine, Request, StepEvent
@@ -34,9 +36,6 @@ def build_model(model: str, tp: Optional[TPGroup] = None, dtype: str = "bf16", d
     """
     tp = tp or TPGroup()
     device = torch.device(device) if device is not None else default_device(tp)
-    if device.type == "cuda":
-        if dtype not in ("bf16", "bfloat16"):
-            raise ValueError("the gfx950 kernels compute in bf16 (optionally fp8 weights)")
     tdtype = _DTYPES[dtype]
     is_dir = os.path.isdir(model)
     if random_init is None:
@@ -45,6 +44,18 @@ def build_model(model: str, tp: Optional[TPGroup] = None, dtype: str = "bf16", d
         cfg = ModelConfig.from_pretrained(model)
     else:
         cfg = get_preset(model)
+    if cfg.layer_specs:
+        # per-layer designs: their kernels run in bf16 or as a true fp32 model (csrc/anytype.h); no fp8, no TP
+        if fp8:
+            raise ValueError(f"{cfg.model_type}: fp8 weights are not supported")
+        if random_init:
+            w = random_timisun_weights(cfg, device=device, dtype=tdtype, seed=seed)
+        else:
+            w = load_timisun_weights(cfg, CheckpointReader(weight_files(model)), device=device, dtype=tdtype)
+        return create_model(cfg, w, tp)
+    if device.type == "cuda":
+        if dtype not in ("bf16", "bfloat16"):
+            raise ValueError("the gfx950 kernels of this family compute in bf16 (optionally fp8 weights)")
     if random_init:
         w = random_weights(cfg, tp.size, tp.rank, device=device, dtype=tdtype, seed=seed, fp8=fp8)
     else:

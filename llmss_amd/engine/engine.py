@@ -144,6 +144,9 @@ class LLMEngine:
                  autotune: Optional[bool] = None, prefill_chunk: Optional[int] = None,
                  kv_dtype: Optional[str] = None):
         self.model = model
+        # the uniform families (DecoderLM) have GEMM plans to tune and TP decode schedules to choose between; a
+        # per-layer design (LayeredLM) shares everything else: scheduler, paged pool, graphs, sampler
+        self._uniform = isinstance(model, DecoderLM)
         if kv_dtype is not None:  # "bf16" (model dtype) or "fp8" (e4m3 rows + per-row scale)
             if kv_dtype not in ("bf16", "fp8"):
                 raise ValueError(f"kv_dtype must be 'bf16' or 'fp8', not {kv_dtype!r}")
@@ -209,18 +212,18 @@ class LLMEngine:
         self.buf = _DecodeBuffers(self.buckets[-1], self.max_blocks, self.device) if self.is_gpu else None
         if self.is_gpu:
             _hip_ops.reserve_workspace(self.device, 64 << 20)
-            for b in self.decode_batch_sizes():
+            for b in self.decode_batch_sizes() if self._uniform else ():
                 nsplit, _ = self._splits(b)
                 if nsplit > 1:
                     _hip_ops._DECODE_WS.get(b, model.plan.nh_l, nsplit, self.cfg.head_dim, self.device)
         if autotune is None:
             autotune = os.environ.get("LLMSS_AUTOTUNE", "1") != "0"
         self.tuned = {}
-        if self.is_gpu and autotune:  # per-shape GEMM plans for every decode bucket (ops/autotune.py)
+        if self.is_gpu and autotune and self._uniform:  # per-shape GEMM plans for every decode bucket (ops/autotune.py)
             from ..ops.autotune import tune_model
 
             self.tuned = tune_model(model, self.decode_batch_sizes())
-        if self.is_gpu and autotune:
+        if self.is_gpu and autotune and self._uniform:
             self._tune_gqa_attention()
         if self.use_graphs and os.environ.get("LLMSS_GRAPHS", "1") == "0":
             self.use_graphs = False
@@ -265,7 +268,7 @@ class LLMEngine:
                 "tbo_min": self.model.tbo_min, "graph_keys": sorted(self.graphs),
                 "decode_schedule": sorted(self.decode_schedule.items()), "rsag_mode": self.model.rsag_mode,
                 "col": [self.model.col_mode, self.model.col_chunks, sorted(self.model.col)],
-                "fp8": any(L.qkv.w_scale is not None for L in self.model.w.layers[:1])}
+                "fp8": self._uniform and any(L.qkv.w_scale is not None for L in self.model.w.layers[:1])}
 
     def _default_buckets(self):
         out, b = [], 1
@@ -549,6 +552,34 @@ class LLMEngine:
         self.stats["tokens"] += len(events)
         return events
 
+    def _step_input(self, batch, ids: np.ndarray, last_idx: Optional[np.ndarray]) -> StepInput:
+        """The StepInput of a scheduled batch (Scheduler.schedule or Scheduler.feed) over its flattened token ids:
+        rows [0, num_decode) are single tokens after a cached prefix, then one portion per prompting sequence
+        (positions ctx - q .. ctx - 1). Block tables and context lengths ride along with every kind of step: models
+        that attend through the paged cache alone (LayeredLM) need them for a first portion as well."""
+        dev = self.device
+        qlens = batch.query_lens.astype(np.int64)
+        ctx = batch.ctx_lens.astype(np.int64)
+        nd = int(batch.num_decode)
+
+        def d(a):
+            return torch.from_numpy(np.ascontiguousarray(a)).to(dev, non_blocking=True)
+
+        bt, cl = d(batch.block_table.astype(np.int32)), d(ctx.astype(np.int32))
+        li = d(np.asarray(last_idx, dtype=np.int64)) if last_idx is not None else None
+        if nd == len(qlens):  # single tokens only
+            return StepInput(kind="decode", input_ids=d(ids), positions=d(batch.positions), slots=d(batch.slots),
+                             block_tables=bt, ctx_lens=cl, max_ctx=self.max_model_len, last_idx=li)
+        ends = np.cumsum(qlens)
+        cu = np.zeros(len(qlens) - nd + 1, dtype=np.int32)
+        cu[1:] = ends[nd:] - (ends[nd - 1] if nd else 0)
+        has_prefix = bool((ctx[nd:] > qlens[nd:]).any())
+        kind = "prefill" if nd == 0 and not has_prefix else "extend"
+        return StepInput(
+            kind=kind, input_ids=d(ids), positions=d(batch.positions), slots=d(batch.slots), cu_seqlens=d(cu),
+            max_seqlen=int(qlens[nd:].max()), last_idx=li, block_tables=bt, ctx_lens=cl, max_ctx=self.max_model_len,
+            num_decode=nd, has_prefix=has_prefix, cu_host=cu if kind == "prefill" else None)
+
     def _extend(self, batch, reqs: List[Request]) -> List[int]:
         """A step with prompt chunks: rows [0, num_decode) are decode tokens, then one chunk per
         prompting sequence (positions ctx - q .. ctx - 1). Returns the tokens sampled for the
@@ -556,24 +587,9 @@ class LLMEngine:
         dev = self.device
         qlens = batch.query_lens.astype(np.int64)
         ctx = batch.ctx_lens.astype(np.int64)
-        nd = int(batch.num_decode)
         ids = np.concatenate([np.asarray(r.all_ids[c - q:c], dtype=np.int64) for r, q, c in zip(reqs, qlens, ctx)])
-        ends = np.cumsum(qlens)
-        cu = np.zeros(len(reqs) - nd + 1, dtype=np.int32)
-        cu[1:] = ends[nd:] - (ends[nd - 1] if nd else 0)
         smp = batch.sample
-        has_prefix = bool((ctx[nd:] > qlens[nd:]).any())
-        kind = "prefill" if nd == 0 and not has_prefix else "extend"
-
-        def d(a):
-            return torch.from_numpy(np.ascontiguousarray(a)).to(dev, non_blocking=True)
-
-        inp = StepInput(
-            kind=kind, input_ids=d(ids), positions=d(batch.positions), slots=d(batch.slots), cu_seqlens=d(cu),
-            max_seqlen=int(qlens[nd:].max()), last_idx=d((ends - 1)[smp]),
-            block_tables=d(batch.block_table.astype(np.int32)) if kind == "extend" else None,
-            ctx_lens=d(ctx.astype(np.int32)) if kind == "extend" else None, max_ctx=self.max_model_len,
-            num_decode=nd, has_prefix=has_prefix, cu_host=cu if kind == "prefill" else None)
+        inp = self._step_input(batch, ids, (np.cumsum(qlens) - 1)[smp])
         reqs = [r for r, f in zip(reqs, smp) if f]
         if not reqs:
             self.model.hidden_states(inp, self.kv)  # prompt chunks only: fill the cache, nothing to sample
@@ -582,6 +598,42 @@ class LLMEngine:
         tok = self._forward_sample(inp, *(torch.from_numpy(a).to(dev) for a in (temp, topk, topp, seeds)),
                                    dist=self._dist_ok(temp, topk))
         return tok.cpu().tolist()
+
+    def replay_step(self, entries: Sequence[tuple], end: Iterable[int] = ()) -> Optional[torch.Tensor]:
+        """One step dictated from outside instead of planned by the scheduler (replaying a recorded schedule):
+        ``entries`` = [(request id, its next token ids, positions among them whose logits are wanted)], all run as
+        ONE batch - portions of prompts beside single tokens - from the cache earlier steps left; a request is
+        admitted at its first entry and may sit out a step. ``end``: requests finished after this step, whose
+        blocks and sequence slot go back to the pool. Nothing is sampled. Returns the fp32 logits [wanted, vocab]
+        in the order of the entries and of their wanted positions (None when nothing is wanted).
+
+        It goes through the engine's own scheduler state (Scheduler.feed: block allocator, slot mapping, block
+        tables), cache and model step, like a planned step; it must not be mixed with pending pipelined decodes."""
+        if self._pending:
+            raise RuntimeError("replay_step: pipelined decode steps are in flight")
+        out = None
+        if entries:
+            rids = [int(e[0]) for e in entries]
+            batch = self.sched.feed(rids, [len(e[1]) for e in entries])
+            order = batch.ids.tolist()
+            toks = {int(e[0]): e[1] for e in entries}
+            qlens = batch.query_lens.astype(np.int64)
+            if [len(toks[r]) for r in order] != qlens.tolist():
+                raise RuntimeError("replay_step: the scheduler's step does not match the entries")
+            start = dict(zip(order, (np.cumsum(qlens) - qlens).tolist()))
+            ids = np.concatenate([np.asarray(toks[r], dtype=np.int64) for r in order])
+            rows = [start[int(e[0])] + int(w) for e in entries for w in e[2]]
+            if any(not 0 <= int(w) < len(e[1]) for e in entries for w in e[2]):
+                raise ValueError("replay_step: a wanted position lies outside its entry")
+            inp = self._step_input(batch, ids, rows if rows else None)
+            if rows:
+                out = self.model(inp, self.kv)[:, : self.cfg.vocab_size].float()
+            else:
+                self.model.hidden_states(inp, self.kv)
+            self.stats["steps"] += 1
+        for rid in end:
+            self.sched.finish(int(rid))
+        return out
 
     def _dist_ok(self, temp, topk) -> bool:
         """Sample this step from vocab-parallel candidates (no [B, V] logits all-gather)?"""

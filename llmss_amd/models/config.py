@@ -15,13 +15,55 @@ Families (``MODEL_REGISTRY`` keys, reference ``custom_modeling/__init__.py:4-7``
 * ``gpt_bigcode`` - LayerNorm, learned positions, MQA (or MHA) fused c_attn, tied head
                     (``gpt_bigcode_modeling.py``).
 * ``llama``       - RMSNorm, half-rotate RoPE, GQA, SwiGLU, untied head.
+* ``timisun``     - per-layer description (``layer_specs``): parallel blocks over an fp32 residual, latent
+                    attention without positions (sliding window, latent rows shared between layers),
+                    mixture-of-experts feed-forward with a shared expert, scaled embedding, tied head.
 """
 from __future__ import annotations
 
 import json
 import os
 from dataclasses import asdict, dataclass, field, replace
-from typing import Any, Dict, Optional
+from typing import Any, Dict, List, Optional
+
+
+@dataclass
+class MixerSpec:
+    """One layer's token mixer. ``latent_attention``: ``heads`` heads of ``dim`` query/key and ``vdim`` value
+    dimensions over a cached latent row of ``kv_rank`` numbers; ``window`` > 0 limits a position to itself and the
+    ``window - 1`` positions before it (0 = every earlier position); ``kv_from`` = index of the layer whose cached
+    latent rows this layer reads instead of projecting its own."""
+    kind: str
+    heads: int
+    dim: int
+    vdim: int
+    kv_rank: int
+    scale: float
+    window: int = 0
+    kv_from: Optional[int] = None
+
+
+@dataclass
+class ExpertSpec:
+    ff: int
+    limit: float
+
+
+@dataclass
+class MoESpec:
+    """Mixture-of-experts feed-forward: ``experts`` experts of which each token uses ``top``; ``shared`` runs for
+    every token."""
+    experts: int
+    top: int
+    expert: ExpertSpec
+    shared: Optional[ExpertSpec] = None
+    kind: str = "moe"
+
+
+@dataclass
+class LayerSpec:
+    mixer: MixerSpec
+    mlp: Optional[MoESpec] = None
 
 
 @dataclass
@@ -54,6 +96,11 @@ class ModelConfig:
     eos_token_id: Optional[int] = None
     pad_token_id: Optional[int] = None
     extra: Dict[str, Any] = field(default_factory=dict)
+    # per-layer designs (layers that differ from each other): one LayerSpec per layer; None for the uniform families
+    layer_specs: Optional[List[LayerSpec]] = None
+    embedding_scale: float = 1.0  # the embedding row is multiplied by this
+    norm_offset: float = 0.0  # norm weights are stored as (w - offset): 1.0 = stored around zero
+    residual_fp32: bool = False  # the residual stream is kept and summed in fp32
 
     # ---------------------------------------------------------------- derived
     @property
@@ -88,6 +135,8 @@ class ModelConfig:
     @classmethod
     def from_hf_dict(cls, d: Dict[str, Any]) -> "ModelConfig":
         mt = d.get("model_type")
+        if mt is None and d.get("architecture") == "Timisun":
+            return _timisun(cls, d)
         common = dict(
             bos_token_id=d.get("bos_token_id"),
             eos_token_id=_first(d.get("eos_token_id")),
@@ -151,6 +200,51 @@ class ModelConfig:
             return cls.from_hf_dict(json.load(f))
 
 
+def _timisun(cls, d: Dict[str, Any]) -> "ModelConfig":
+    """``{"architecture": "Timisun", "vocab", "width", "embedding": {"scale"}, "norm": {"eps"}, "layers": [{"type",
+    "mixer": {"heads", "dim", "vdim", "kv_rank", "scale", "mask": {"size"}, "kv_from"}, "mlp": {"kind": "moe",
+    "router": {"experts", "top"}, "expert": {"ff", "limit"}, "shared": {"ff", "limit"}} | null}]}``."""
+    specs: List[LayerSpec] = []
+    for i, L in enumerate(d["layers"]):
+        if L.get("type") != "latent_attention":
+            raise ValueError(f"Timisun layer {i}: unsupported mixer type {L.get('type')!r}")
+        m = L["mixer"]
+        mask = m.get("mask") or {}
+        kv_from = m.get("kv_from")
+        mixer = MixerSpec("latent_attention", int(m["heads"]), int(m["dim"]), int(m["vdim"]), int(m["kv_rank"]),
+                          float(m["scale"]), int(mask.get("size") or 0), None if kv_from is None else int(kv_from))
+        if mixer.kv_from is not None:
+            j = mixer.kv_from
+            if not 0 <= j < i or specs[j].mixer.kv_from is not None or specs[j].mixer.kv_rank != mixer.kv_rank:
+                raise ValueError(f"Timisun layer {i}: kv_from {j} must name an earlier layer that projects its own "
+                                 f"latent rows of the same rank")
+        mlp = None
+        f = L.get("mlp")
+        if f is not None:
+            if f.get("kind", "moe") != "moe":
+                raise ValueError(f"Timisun layer {i}: unsupported feed-forward kind {f.get('kind')!r}")
+            sh = f.get("shared")
+            mlp = MoESpec(int(f["router"]["experts"]), int(f["router"]["top"]),
+                          ExpertSpec(int(f["expert"]["ff"]), float(f["expert"]["limit"])),
+                          None if sh is None else ExpertSpec(int(sh["ff"]), float(sh["limit"])))
+            if not 1 <= mlp.top <= mlp.experts:
+                raise ValueError(f"Timisun layer {i}: top {mlp.top} of {mlp.experts} experts")
+        specs.append(LayerSpec(mixer, mlp))
+    if not specs:
+        raise ValueError("Timisun: no layers")
+    return cls(
+        model_type="timisun", vocab_size=int(d["vocab"]), hidden_size=int(d["width"]), num_layers=len(specs),
+        num_heads=max(s.mixer.heads for s in specs), num_kv_heads=1, head_dim=max(s.mixer.kv_rank for s in specs),
+        intermediate_size=max([s.mlp.expert.ff for s in specs if s.mlp] or [0]),
+        max_position_embeddings=1 << 20,  # the design has no positional limit of its own
+        norm="rmsnorm", norm_eps=float(d["norm"]["eps"]), activation="glu_clamp", position="none", rotary_dim=0,
+        parallel_block=True, tie_word_embeddings=True, layer_specs=specs,
+        embedding_scale=float((d.get("embedding") or {}).get("scale", 1.0)), norm_offset=1.0, residual_fp32=True,
+        bos_token_id=d.get("bos_token_id"), eos_token_id=_first(d.get("eos_token_id")),
+        pad_token_id=d.get("pad_token_id"),
+    )
+
+
 def _first(x):
     if isinstance(x, (list, tuple)):
         return x[0] if x else None
@@ -209,6 +303,20 @@ _PRESETS: Dict[str, Dict[str, Any]] = {
     "tiny-llama": dict(model_type="llama", hidden_size=64, num_hidden_layers=2, num_attention_heads=4,
                        num_key_value_heads=2, intermediate_size=160, vocab_size=211,
                        max_position_embeddings=128),
+    # per-layer design: 3 layers, the last reading layer 0's latent rows; one layer without a feed-forward
+    "tiny-timisun": dict(architecture="Timisun", vocab=211, width=48, embedding=dict(scale=4.0), norm=dict(eps=1e-5),
+                         layers=[
+                             dict(type="latent_attention",
+                                  mixer=dict(heads=3, dim=8, vdim=12, kv_rank=24, scale=0.3, mask=dict(size=9)),
+                                  mlp=dict(kind="moe", router=dict(experts=5, top=2), expert=dict(ff=20, limit=3.0),
+                                           shared=dict(ff=12, limit=1.5))),
+                             dict(type="latent_attention",
+                                  mixer=dict(heads=2, dim=16, vdim=8, kv_rank=16, scale=0.25), mlp=None),
+                             dict(type="latent_attention",
+                                  mixer=dict(heads=3, dim=8, vdim=12, kv_rank=24, scale=0.3, mask=dict(size=5),
+                                             kv_from=0),
+                                  mlp=dict(kind="moe", router=dict(experts=4, top=1), expert=dict(ff=16, limit=2.0))),
+                         ]),
     # TP up to 8 (16 q / kv heads: 2 per rank at TP=8, as Llama-2-7B's 32 give 4)
     "tiny-llama16h": dict(model_type="llama", hidden_size=256, num_hidden_layers=2, num_attention_heads=16,
                           num_key_value_heads=16, intermediate_size=512, vocab_size=211,

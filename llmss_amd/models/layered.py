@@ -1,0 +1,197 @@
+"""Decoder whose layers are described one by one (``ModelConfig.layer_specs``) over an fp32 residual stream.
+
+The uniform families run through :class:`~llmss_amd.models.decoder.DecoderLM`; a per-layer design (Timisun) runs
+through :class:`LayeredLM`, which offers the engine the same surface (``hidden_states`` / ``logits`` over a
+:class:`StepInput`, ``allocate_kv_cache``, ``kv_bytes_per_block``, ``plan``) and so shares its scheduler, paged
+cache pool, decode graphs and sampler. Each layer is a parallel block
+
+    h = norm(x) ;  x <- x + (mixer(h) + ffn(h))          x fp32, norm weight stored around zero
+
+with the mixer and the feed-forward looked up by kind (``MIXERS`` / ``FFNS``), so another design can combine the
+same mechanisms with other constants or add its own beside them.
+
+Mixer ``latent_attention`` (ops: linear_f, latent_norm_cache, head_absorb, latent_attn, head_expand): the layer
+caches one RMS-normed latent row c per token in its paged cache ([blocks, block_size, kv_rank], the step's slots)
+and attends with the key projection absorbed into the query: qa_h = W_uk_h^T q_h, p = softmax(scale qa_h . c_j)
+over the causal (optionally windowed) keys, out = W_o concat_h(W_uv_h sum_j p_j c_j). A layer with ``kv_from``
+projects no latent of its own and reads the named layer's cache with its own W_uk / W_uv.
+
+Feed-forward ``moe`` (ops: linear_f -> fp32 router logits, moe_route, moe_experts, glu_clamp): sigmoid scores, the
+choice made on score + correction, weights = chosen scores normalised; experts and the shared expert use the clamped
+gated activation g * sigmoid(1.702 g) * (u + 1).
+"""
+from __future__ import annotations
+
+from typing import List, Optional
+
+import torch
+
+from .. import ops
+from ..parallel.dist import TPGroup
+from .config import ModelConfig
+from .decoder import StepInput
+from .weights import ModelWeights, ShardPlan
+
+GLU_ALPHA = 1.702  # the gate's sigmoid slope of the clamped gated activation
+
+
+class LatentAttention:
+    """Mixer ``latent_attention``."""
+
+    @staticmethod
+    def cache_row(spec) -> Optional[int]:
+        """Numbers cached per token by a layer of this kind (None: it reads another layer's cache)."""
+        return spec.kv_rank if spec.kv_from is None else None
+
+    @staticmethod
+    def forward(model: "LayeredLM", i: int, W, spec, h, inp: StepInput, cu, caches):
+        dt = model.dtype
+        H, dim, R = spec.heads, spec.dim, spec.kv_rank
+        qc = ops.linear_f(h, W.qc, dt)  # [T, H * dim (+ R)]: queries, then this layer's raw latent
+        cache = caches[i if spec.kv_from is None else spec.kv_from][0]
+        if W.own_kv:
+            ops.latent_norm_cache(qc, H * dim, R, W.kv_norm, model.cfg.norm_eps, cache, inp.slots)
+        qa = ops.head_absorb(qc, W.uk, H, dim)
+        o = ops.latent_attn(qa, cache, inp.block_tables, cu, inp.ctx_lens, spec.window, spec.scale)
+        return ops.linear_f(ops.head_expand(o, W.uv, dt), W.o, dt)
+
+
+class MoEFeedForward:
+    """Feed-forward ``moe``."""
+
+    @staticmethod
+    def forward(model: "LayeredLM", W, spec, h):
+        dt = model.dtype
+        z = ops.linear_f(h, W.router, torch.float32)
+        idx, wts = ops.moe_route(z, W.correction, spec.top)
+        sh = None
+        if W.shared_gu is not None:
+            gu = ops.linear_f(h, W.shared_gu, dt)
+            sh = ops.linear_f(ops.glu_clamp(gu, spec.shared.ff, spec.shared.limit, GLU_ALPHA), W.shared_down, dt)
+        return ops.moe_experts(h, idx, wts, W.gate, W.up, W.down, spec.expert.limit, GLU_ALPHA, shared=sh)
+
+
+MIXERS = {"latent_attention": LatentAttention}
+FFNS = {"moe": MoEFeedForward}
+
+
+class LayeredLM:
+    def __init__(self, cfg: ModelConfig, weights: ModelWeights, tp: Optional[TPGroup] = None):
+        if not cfg.layer_specs:
+            raise ValueError("LayeredLM needs a config with layer_specs")
+        self.cfg = cfg
+        self.w = weights
+        self.tp = tp or TPGroup()
+        if self.tp.size != 1:
+            raise NotImplementedError(f"{cfg.model_type}: tensor parallelism is not implemented for per-layer designs")
+        for s in cfg.layer_specs:
+            if s.mixer.kind not in MIXERS:
+                raise ValueError(f"unknown mixer kind {s.mixer.kind!r}")
+            if s.mlp is not None and s.mlp.kind not in FFNS:
+                raise ValueError(f"unknown feed-forward kind {s.mlp.kind!r}")
+        self.plan = ShardPlan(1, 0, cfg.num_heads, 0, 1, cfg.intermediate_size, weights.head.w.shape[0])
+        # what the engine asks of every model: no TP decode schedules, no fp8 cache rows here
+        self.kv_fp8 = False
+        self.tbo_min = 0
+        self.rsag_mode = self.col_mode = "0"
+        self.rsag: set = set()
+        self.col: set = set()
+        self.col_chunks = 0
+        self.overlap_rows = None
+        self.bucket_bytes = 0
+        self.gqa_mfma: set = set()
+        self._cu_decode = {}
+        self.tap = None  # tap(i, x): called with the fp32 residual after layer i (debugging, tests)
+
+    @property
+    def device(self):
+        return self.w.wte.device
+
+    @property
+    def dtype(self):
+        return self.w.wte.dtype
+
+    def overlap_split(self, B: int) -> int:
+        return 0
+
+    # --------------------------------------------------------------------------------- cache
+    def _cache_rows(self) -> List[Optional[int]]:
+        return [MIXERS[s.mixer.kind].cache_row(s.mixer) for s in self.cfg.layer_specs]
+
+    def kv_bytes_per_block(self, block_size: int) -> int:
+        return sum(block_size * r * self.w.wte.element_size() for r in self._cache_rows() if r)
+
+    def allocate_kv_cache(self, num_blocks: int, block_size: int):
+        """One (rows, None) pair per layer; a layer that reads another layer's rows holds that layer's pair."""
+        caches: list = []
+        for s, r in zip(self.cfg.layer_specs, self._cache_rows()):
+            if r:
+                caches.append((torch.zeros(num_blocks, block_size, r, dtype=self.dtype, device=self.device), None))
+            else:
+                caches.append(caches[s.mixer.kv_from])
+        return caches
+
+    # ---------------------------------------------------------------------------- forward
+    def decode_cu(self, B: int, device) -> torch.Tensor:
+        cu = self._cu_decode.get((B, str(device)))
+        if cu is None:
+            cu = self._cu_decode[(B, str(device))] = torch.arange(B + 1, dtype=torch.int32, device=device)
+        return cu
+
+    def _cu(self, inp: StepInput) -> torch.Tensor:
+        """Row boundaries of every sequence of the step, single-token rows first (the order of block_tables)."""
+        dev = inp.input_ids.device
+        if inp.kind == "decode":
+            return self.decode_cu(inp.input_ids.shape[0], dev)
+        if inp.num_decode:
+            return torch.cat([torch.arange(inp.num_decode, dtype=torch.int32, device=dev),
+                              inp.cu_seqlens.to(torch.int32) + inp.num_decode])
+        return inp.cu_seqlens
+
+    def hidden_states(self, inp: StepInput, kv_caches) -> torch.Tensor:
+        if inp.block_tables is None or inp.ctx_lens is None or kv_caches[0][0] is None:
+            raise ValueError(f"{self.cfg.model_type} attends through its paged cache: the step needs block tables, "
+                             f"context lengths and a cache (a cache-less recompute step is not supported)")
+        cfg, w = self.cfg, self.w
+        eps, off, dt = cfg.norm_eps, cfg.norm_offset, self.dtype
+        cu = self._cu(inp)
+        x = ops.embed_scaled(inp.input_ids, w.wte, cfg.embedding_scale)
+        a = f = None
+        for i, (L, spec) in enumerate(zip(w.layers, cfg.layer_specs)):
+            h = ops.resid_add_norm(x, a, f, L.norm1, off, eps, dt)
+            if self.tap is not None and i:
+                self.tap(i - 1, x)
+            a = MIXERS[spec.mixer.kind].forward(self, i, L.mix, spec.mixer, h, inp, cu, kv_caches)
+            f = FFNS[spec.mlp.kind].forward(self, L.mlp, spec.mlp, h) if spec.mlp is not None else None
+        h = ops.resid_add_norm(x, a, f, w.lnf_w, off, eps, dt)
+        if self.tap is not None:
+            self.tap(len(w.layers) - 1, x)
+        return h
+
+    @property
+    def vocab_lo(self) -> int:
+        return 0
+
+    def local_logits(self, h: torch.Tensor) -> torch.Tensor:
+        return ops.linear_f(h, self.w.head.w, self.dtype)
+
+    def logits(self, h: torch.Tensor) -> torch.Tensor:
+        """[B, H] -> [B, V padded to 16] against the embedding table itself (no embedding scale)."""
+        return self.local_logits(h)
+
+    def forward(self, inp: StepInput, kv_caches) -> torch.Tensor:
+        h = self.hidden_states(inp, kv_caches)
+        if inp.last_idx is not None:
+            h = h.index_select(0, inp.last_idx)
+        return self.logits(h)
+
+    __call__ = forward
+
+
+def create_model(cfg: ModelConfig, weights: ModelWeights, tp: Optional[TPGroup] = None):
+    """The model class of a config: per-layer designs -> LayeredLM, the uniform families -> DecoderLM."""
+    if cfg.layer_specs:
+        return LayeredLM(cfg, weights, tp)
+    from .decoder import DecoderLM
+
+    return DecoderLM(cfg, weights, tp)

@@ -150,6 +150,9 @@ def _tensors(mw: ModelWeights):
     if mw.wpe is not None:
         yield mw.wpe
     for L in mw.layers:
+        if hasattr(L, "tensors"):  # per-layer designs describe themselves
+            yield from L.tensors()
+            continue
         for t in (L.ln1_w, L.ln1_b, L.ln2_w, L.ln2_b):
             if t is not None:
                 yield t
@@ -527,3 +530,175 @@ def shard_cache_path(root: str, model_dir: str, files: List[str], tp: int, rank:
         h.update(f"{os.path.basename(f)}:{st.st_size}:{int(st.st_mtime)}".encode())
     tag = str(dtype).replace("torch.", "") + ("-fp8" if fp8 else "")
     return os.path.join(root, h.hexdigest()[:16], f"tp{tp}-r{rank}-{tag}.safetensors")
+
+
+# ------------------------------------------------------------------------------ per-layer designs (Timisun)
+@dataclass
+class LatentAttnWeights:
+    """Latent attention: ``qc`` [heads * dim (+ kv_rank), H] is the query projection followed, in a layer that
+    projects its own latent rows (``own_kv``), by the latent down-projection - one GEMM for both; ``kv_norm``
+    [kv_rank] the latent's plain RMS-norm weight; ``uk`` [heads * dim, kv_rank] and ``uv`` [heads * vdim, kv_rank]
+    the per-head key / value up-projections; ``o`` [H, heads * vdim]."""
+    qc: torch.Tensor
+    own_kv: bool
+    kv_norm: Optional[torch.Tensor]
+    uk: torch.Tensor
+    uv: torch.Tensor
+    o: torch.Tensor
+
+    def tensors(self):
+        return [t for t in (self.qc, self.kv_norm, self.uk, self.uv, self.o) if t is not None]
+
+
+@dataclass
+class MoEWeights:
+    """Experts stacked: ``gate`` / ``up`` [E, F, H], ``down`` [E, H, F]; ``router`` [E, H]; ``correction`` fp32 [E]
+    (added to the scores for the choice only); the shared expert as one gate | up matrix ``shared_gu`` [2 Fs, H]
+    and ``shared_down`` [H, Fs]."""
+    router: torch.Tensor
+    correction: Optional[torch.Tensor]
+    gate: torch.Tensor
+    up: torch.Tensor
+    down: torch.Tensor
+    shared_gu: Optional[torch.Tensor] = None
+    shared_down: Optional[torch.Tensor] = None
+
+    def tensors(self):
+        return [t for t in (self.router, self.correction, self.gate, self.up, self.down, self.shared_gu,
+                            self.shared_down) if t is not None]
+
+
+@dataclass
+class BlockWeights:
+    """One parallel block of a per-layer design: a single norm feeding the mixer and the feed-forward."""
+    norm1: torch.Tensor
+    mix: LatentAttnWeights
+    mlp: Optional[MoEWeights]
+
+    def tensors(self):
+        return [self.norm1] + self.mix.tensors() + (self.mlp.tensors() if self.mlp else [])
+
+
+def _tied_head(cfg: ModelConfig, wte: torch.Tensor, device, dtype):
+    """One device table [V padded to 16, H]: the embedding is its first V rows, the head the whole of it."""
+    vp = math.ceil(cfg.vocab_size / 16) * 16
+    table = torch.zeros(vp, cfg.hidden_size, dtype=dtype, device=device)
+    table[:cfg.vocab_size].copy_(wte.to(device=device, dtype=dtype))
+    return table[:cfg.vocab_size], Linear(table)
+
+
+def _timisun_finish(cfg: ModelConfig, get, device, dtype) -> ModelWeights:
+    """``get(name)`` returns the checkpoint tensor of that name (CPU); tensor names as in the checkpoint:
+    ``embed``, ``final.norm``, ``l<i>.norm1``, ``l<i>.mix.{q,dkv,dkv.norm,uk,uv,o}``,
+    ``l<i>.mlp.{router,correction,e<k>.{gate,up,down},shared.{gate,up,down}}``."""
+    def dev(t, dt=dtype):
+        return t.to(device=device, dtype=dt).contiguous()
+
+    layers = []
+    for i, spec in enumerate(cfg.layer_specs):
+        p = f"l{i}."
+        mx = spec.mixer
+        own = mx.kv_from is None
+        q = get(p + "mix.q")
+        mix = LatentAttnWeights(
+            qc=dev(torch.cat([q, get(p + "mix.dkv")], 0) if own else q), own_kv=own,
+            kv_norm=dev(get(p + "mix.dkv.norm")) if own else None,
+            uk=dev(get(p + "mix.uk")), uv=dev(get(p + "mix.uv")), o=dev(get(p + "mix.o")))
+        want = {"qc": (mx.heads * mx.dim + (mx.kv_rank if own else 0), cfg.hidden_size),
+                "uk": (mx.heads * mx.dim, mx.kv_rank), "uv": (mx.heads * mx.vdim, mx.kv_rank),
+                "o": (cfg.hidden_size, mx.heads * mx.vdim)}
+        for nm, shp in want.items():
+            if tuple(getattr(mix, nm).shape) != shp:
+                raise ValueError(f"layer {i}: {nm} has shape {tuple(getattr(mix, nm).shape)}, the config says {shp}")
+        mlp = None
+        if spec.mlp is not None:
+            f, m = spec.mlp, p + "mlp."
+            E = f.experts
+            sh_gu = sh_down = None
+            if f.shared is not None:
+                sh_gu = dev(torch.cat([get(m + "shared.gate"), get(m + "shared.up")], 0))
+                sh_down = dev(get(m + "shared.down"))
+            mlp = MoEWeights(
+                router=dev(get(m + "router")), correction=dev(get(m + "correction"), torch.float32),
+                gate=dev(torch.stack([get(f"{m}e{k}.gate") for k in range(E)])),
+                up=dev(torch.stack([get(f"{m}e{k}.up") for k in range(E)])),
+                down=dev(torch.stack([get(f"{m}e{k}.down") for k in range(E)])),
+                shared_gu=sh_gu, shared_down=sh_down)
+            if tuple(mlp.gate.shape) != (E, f.expert.ff, cfg.hidden_size):
+                raise ValueError(f"layer {i}: expert gate {tuple(mlp.gate.shape)} does not fit the config")
+        layers.append(BlockWeights(dev(get(p + "norm1")), mix, mlp))
+    wte, head = _tied_head(cfg, get("embed"), device, dtype)
+    return ModelWeights(wte=wte, wpe=None, layers=layers, lnf_w=dev(get("final.norm")), lnf_b=None, head=head)
+
+
+def load_timisun_weights(cfg: ModelConfig, reader, device="cpu", dtype=torch.bfloat16) -> ModelWeights:
+    return _timisun_finish(cfg, lambda n: reader.get(n), device, dtype)
+
+
+def random_timisun_weights(cfg: ModelConfig, device="cpu", dtype=torch.bfloat16, seed: int = 0) -> ModelWeights:
+    """Random-init weights of a per-layer (Timisun) config: projections ~ N(0, 1 / fan_in), norm weights and the
+    router's correction small around zero, values rounded to bf16 (so a bf16 and an fp32 run hold the same model)."""
+    return _timisun_finish(cfg, _timisun_random(cfg, seed), device, dtype)
+
+
+def timisun_state_dict(cfg: ModelConfig, seed: int = 0) -> Dict[str, torch.Tensor]:
+    """The random weights of :func:`random_timisun_weights` under their checkpoint names (bf16; tests, examples)."""
+    get = _timisun_random(cfg, seed)
+    names = ["embed", "final.norm"]
+    for i, spec in enumerate(cfg.layer_specs):
+        p = f"l{i}."
+        names += [p + "norm1", p + "mix.q", p + "mix.uk", p + "mix.uv", p + "mix.o"]
+        if spec.mixer.kv_from is None:
+            names += [p + "mix.dkv", p + "mix.dkv.norm"]
+        if spec.mlp is not None:
+            names += [p + "mlp.router", p + "mlp.correction"]
+            for k in range(spec.mlp.experts):
+                names += [f"{p}mlp.e{k}.{n}" for n in ("gate", "up", "down")]
+            if spec.mlp.shared is not None:
+                names += [f"{p}mlp.shared.{n}" for n in ("gate", "up", "down")]
+    return {n: get(n).to(torch.bfloat16) for n in names}
+
+
+def _timisun_random(cfg: ModelConfig, seed: int):
+    import zlib
+
+    W = cfg.hidden_size
+
+    def shape_of(name: str):
+        if name == "embed":
+            return (cfg.vocab_size, W), 1.0 / cfg.embedding_scale
+        if name == "final.norm":
+            return (W,), 0.1
+        i = int(name[1:name.index(".")])
+        spec, rest = cfg.layer_specs[i], name[name.index(".") + 1:]
+        mx, f = spec.mixer, spec.mlp
+        if rest == "norm1":
+            return (W,), 0.1
+        if rest == "mix.q":
+            return (mx.heads * mx.dim, W), W ** -0.5
+        if rest == "mix.dkv":
+            return (mx.kv_rank, W), W ** -0.5
+        if rest == "mix.dkv.norm":
+            return (mx.kv_rank,), None  # around one
+        if rest == "mix.uk":
+            return (mx.heads * mx.dim, mx.kv_rank), mx.kv_rank ** -0.5 / max(mx.scale, 1e-6) / mx.dim ** 0.5
+        if rest == "mix.uv":
+            return (mx.heads * mx.vdim, mx.kv_rank), mx.kv_rank ** -0.5
+        if rest == "mix.o":
+            return (W, mx.heads * mx.vdim), (mx.heads * mx.vdim) ** -0.5
+        if rest == "mlp.router":
+            return (f.experts, W), W ** -0.5
+        if rest == "mlp.correction":
+            return (f.experts,), 0.1
+        part = rest.split(".")[-1]
+        e = f.shared if ".shared." in rest else f.expert
+        return ((W, e.ff), e.ff ** -0.5) if part == "down" else ((e.ff, W), W ** -0.5)
+
+    def get(name: str) -> torch.Tensor:
+        g = torch.Generator()
+        g.manual_seed((seed * 1000003 + zlib.crc32(name.encode())) & 0x7FFFFFFF)
+        shp, std = shape_of(name)
+        t = torch.randn(*shp, generator=g, dtype=torch.float32)
+        t = 1.0 + 0.1 * t if std is None else t * std
+        return t.to(torch.bfloat16).float()
+    return get

@@ -149,3 +149,26 @@ def quant_fp8_rows(w):
     if w.is_cuda:
         return _hip().quant_fp8_rows(w)
     return ref.quant_fp8_rows(w)
+
+
+# ------------------------------------------------- fp32 residual stream / latent attention / mixture of experts
+def _route(name):
+    def op(first, *a, **kw):
+        if first.is_cuda:
+            return getattr(_hip(), name)(first, *a, **kw)
+        return getattr(ref, name)(first, *a, **kw)
+    op.__name__ = name
+    op.__doc__ = getattr(ref, name).__doc__
+    return op
+
+
+embed_scaled = _route("embed_scaled")
+resid_add_norm = _route("resid_add_norm")
+linear_f = _route("linear_f")
+head_absorb = _route("head_absorb")
+head_expand = _route("head_expand")
+latent_norm_cache = _route("latent_norm_cache")
+latent_attn = _route("latent_attn")
+glu_clamp = _route("glu_clamp")
+moe_route = _route("moe_route")
+moe_experts = _route("moe_experts")

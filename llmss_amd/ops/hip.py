@@ -774,3 +774,202 @@ def sample(logits, temperature, top_k, top_p, seeds, vocab: Optional[int] = None
     lib().sample(logits.data_ptr(), logits.stride(0), logits.dtype == torch.float32, B, V, _ptr(temperature),
                  _ptr(top_k), _ptr(top_p), _ptr(seeds), y.data_ptr(), _ptr(out2), _stream())
     return y
+
+
+# ------------------------------------------------- fp32 residual stream / latent attention / mixture of experts
+# Kernels that run in either storage type (csrc/anytype.h): bf16 in serving precision, fp32 as a true 32-bit model.
+_DT = {torch.bfloat16: 0, torch.float32: 1}
+
+
+def _dt(t: torch.Tensor, name: str) -> int:
+    _check(t.is_cuda and t.device.index == torch.cuda.current_device(), f"{name} must be on the current GPU")
+    _check(t.dtype in _DT, f"{name} must be bfloat16 or float32, got {t.dtype}")
+    return _DT[t.dtype]
+
+
+def _rows(t: torch.Tensor, name: str, cols: Optional[int] = None, dtype=None):
+    _check(t.dim() == 2 and t.stride(1) == 1, f"{name} must be 2-D with contiguous rows")
+    if cols is not None:
+        _check(t.shape[1] == cols, f"{name} has {t.shape[1]} columns, expected {cols}")
+    if dtype is not None:
+        _check(t.dtype == dtype, f"{name} must be {dtype}, got {t.dtype}")
+    _check(t.is_cuda and t.device.index == torch.cuda.current_device(), f"{name} must be on the current GPU")
+
+
+def embed_scaled(ids, table, scale):
+    T = ids.numel()
+    V, H = table.shape
+    _check(ids.dtype == torch.int64 and ids.is_contiguous() and ids.is_cuda, "ids must be contiguous int64 cuda")
+    _check(table.is_contiguous(), "embedding table contiguous")
+    x = torch.empty(T, H, dtype=torch.float32, device=table.device)
+    lib().embed_scaled(ids.data_ptr(), table.data_ptr(), x.data_ptr(), T, H, V, float(scale), _dt(table, "table"),
+                       _stream())
+    return x
+
+
+def resid_add_norm(x, a, b, w, woff, eps, out_dtype, want_y=True):
+    T, H = x.shape
+    _rows(x, "x", dtype=torch.float32)
+    _check(x.is_contiguous(), "x contiguous")
+    if a is not None:
+        _rows(a, "a", H, out_dtype)
+        _check(a.shape[0] == T, "a rows")
+    if b is not None:
+        _rows(b, "b", H, torch.float32)
+        _check(b.shape[0] == T, "b rows")
+    y = None
+    if want_y:
+        _check(w.dtype == out_dtype and w.is_contiguous() and w.numel() == H, "norm weight")
+        y = torch.empty(T, H, dtype=out_dtype, device=x.device)
+    _check(out_dtype in _DT, "out dtype bf16 / fp32")
+    lib().resid_add_norm(x.data_ptr(), _ptr(a), a.stride(0) if a is not None else 0, _ptr(b),
+                         b.stride(0) if b is not None else 0, _ptr(w) if want_y else 0, float(woff), float(eps),
+                         _ptr(y), H, T, H, _DT[out_dtype], _stream())
+    return y
+
+
+def gemm_any(A, B, C, M, N, K, batch, sAb, sAm, sBb, sBn, sBk, sCb, sCm):
+    """C[b][m][n] = sum_k A[b][m][k] B[b][n][k] over element strides (csrc/gemm_any.hip); the caller has checked that
+    every index stays inside its tensor."""
+    lib().gemm_any(A.data_ptr(), B.data_ptr(), C.data_ptr(), int(M), int(N), int(K), int(batch), int(sAb), int(sAm),
+                   int(sBb), int(sBn), int(sBk), int(sCb), int(sCm), _dt(A, "A"), _dt(B, "B"), _dt(C, "C"), _stream())
+    return C
+
+
+def _mfma_ok(x, w, out_dtype) -> bool:
+    """Can the bf16 MFMA GEMM (csrc/gemm.hip) take this product? bf16 everywhere, K % 16, N % 8, 16-B aligned rows."""
+    return (x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and out_dtype == torch.bfloat16
+            and w.is_contiguous() and x.shape[1] % 16 == 0 and w.shape[0] % 8 == 0 and x.stride(1) == 1
+            and x.data_ptr() % 16 == 0 and (x.stride(0) * 2) % 16 == 0 and w.data_ptr() % 16 == 0)
+
+
+def linear_f(x, w, out_dtype):
+    """x [M, K] . w [N, K]^T -> [M, N] in ``out_dtype`` with fp32 accumulation: the MFMA GEMM where it applies,
+    else the strided VALU GEMM (fp32 storage, fp32 output, odd shapes)."""
+    M, K = x.shape
+    N = w.shape[0]
+    _rows(x, "x")
+    _rows(w, "w", K)
+    _check(w.is_contiguous(), "w contiguous")
+    if M == 0:
+        return torch.empty(0, N, dtype=out_dtype, device=x.device)
+    if _mfma_ok(x, w, out_dtype):
+        return linear(x, w)
+    y = torch.empty(M, N, dtype=out_dtype, device=x.device)
+    return gemm_any(x, w, y, M, N, K, 1, 0, x.stride(0), 0, K, 1, 0, N)
+
+
+def head_absorb(q, uk, H, dim):
+    T = q.shape[0]
+    R = uk.shape[1]
+    _rows(q, "q")
+    _check(q.shape[1] >= H * dim, "q too narrow")
+    _rows(uk, "uk")
+    _check(uk.is_contiguous() and uk.shape[0] == H * dim, "uk [H * dim, R]")
+    qa = torch.empty(T, H, R, dtype=torch.float32, device=q.device)
+    if T:
+        # batch = head: A(t, d) = q[t, h * dim + d]; B(r, d) = uk[h * dim + d, r]
+        gemm_any(q, uk, qa, T, R, dim, H, dim, q.stride(0), dim * R, 1, R, R, H * R)
+    return qa
+
+
+def head_expand(o, uv, out_dtype):
+    T, H, R = o.shape
+    _check(o.is_contiguous() and o.dtype == torch.float32 and o.is_cuda, "o fp32 [T, H, R] contiguous")
+    _rows(uv, "uv", R)
+    _check(uv.is_contiguous() and uv.shape[0] % H == 0, "uv [H * vdim, R]")
+    vd = uv.shape[0] // H
+    y = torch.empty(T, H * vd, dtype=out_dtype, device=o.device)
+    if T:
+        # batch = head: A(t, r) = o[t, h, r]; B(v, r) = uv[h * vd + v, r]; C(t, v) = y[t, h * vd + v]
+        gemm_any(o, uv, y, T, vd, R, H, R, H * R, vd * R, R, 1, vd, H * vd)
+    return y
+
+
+def latent_norm_cache(src, off, R, w, eps, cache, slots):
+    T = src.shape[0]
+    _rows(src, "src")
+    _check(0 <= off and off + R <= src.shape[1], "latent columns outside src")
+    _check(cache.dtype == src.dtype and cache.is_contiguous() and cache.dim() == 3 and cache.shape[2] == R,
+           "latent cache [blocks, block_size, R] in the model's storage type")
+    _check(w.dtype == src.dtype and w.is_contiguous() and w.numel() == R, "latent norm weight")
+    _check(slots.dtype == torch.int64 and slots.is_contiguous() and slots.numel() == T and slots.is_cuda, "slots")
+    lib().latent_norm_cache(src.data_ptr(), src.stride(0), int(off), w.data_ptr(), float(eps), cache.data_ptr(),
+                            slots.data_ptr(), T, R, _dt(src, "src"), _stream())
+
+
+def latent_attn(qa, cache, block_tables, cu_q, ctx_lens, window, scale):
+    T, H, R = qa.shape
+    _check(qa.is_contiguous() and qa.dtype == torch.float32 and qa.is_cuda, "qa fp32 [T, H, R] contiguous")
+    _check(cache.is_contiguous() and cache.dim() == 3 and cache.shape[2] == R, "latent cache [blocks, block_size, R]")
+    B = cu_q.numel() - 1
+    for t, nm in ((cu_q, "cu_q"), (ctx_lens, "ctx_lens"), (block_tables, "block_tables")):
+        _check(t.dtype == torch.int32 and t.is_contiguous() and t.is_cuda, f"{nm} must be contiguous int32 cuda")
+    _check(ctx_lens.numel() >= B and block_tables.dim() == 2 and block_tables.shape[0] >= B, "batch sizes")
+    _check(R <= 512, "latent rank above 512")
+    out = torch.empty(T, H, R, dtype=torch.float32, device=qa.device)
+    lib().latent_attn(qa.data_ptr(), H * R, cache.data_ptr(), block_tables.data_ptr(), block_tables.shape[1],
+                      cu_q.data_ptr(), ctx_lens.data_ptr(), out.data_ptr(), H * R, T, B, H, R, cache.shape[1],
+                      int(window), float(scale), _dt(cache, "cache"), _stream())
+    return out
+
+
+def glu_clamp(gu, F, limit, alpha):
+    T = gu.shape[0]
+    _rows(gu, "gu")
+    _check(gu.shape[1] >= 2 * F, "gate | up too narrow")
+    out = torch.empty(T, F, dtype=gu.dtype, device=gu.device)
+    lib().glu_clamp(gu.data_ptr(), gu.stride(0), out.data_ptr(), F, T, F, float(limit), float(alpha), _dt(gu, "gu"),
+                    _stream())
+    return out
+
+
+def moe_route(z, corr, top):
+    T, E = z.shape
+    _rows(z, "z", dtype=torch.float32)
+    _check(z.is_contiguous(), "router logits contiguous")
+    _check(1 <= top <= E and E <= 4096, "1 <= top <= experts <= 4096")
+    if corr is not None:
+        _check(corr.dtype == torch.float32 and corr.is_contiguous() and corr.numel() == E and corr.is_cuda,
+               "correction fp32 [E]")
+    idx = torch.empty(T, top, dtype=torch.int32, device=z.device)
+    wts = torch.empty(T, top, dtype=torch.float32, device=z.device)
+    lib().moe_route(z.data_ptr(), _ptr(corr), idx.data_ptr(), wts.data_ptr(), T, E, top, _stream())
+    return idx, wts
+
+
+def moe_experts(h, idx, wts, gate, up, down, limit, alpha, shared=None):
+    T, K = h.shape
+    E, F, _ = gate.shape
+    N = down.shape[1]
+    top = idx.shape[1]
+    dt = _dt(h, "h")
+    _rows(h, "h")
+    for t, nm, shp in ((gate, "gate", (E, F, K)), (up, "up", (E, F, K)), (down, "down", (E, N, F))):
+        _check(t.dtype == h.dtype and t.is_contiguous() and tuple(t.shape) == shp and t.is_cuda, f"{nm} {shp}")
+    _check(idx.dtype == torch.int32 and idx.is_contiguous() and idx.shape == (T, top) and idx.is_cuda, "idx")
+    _check(wts.dtype == torch.float32 and wts.is_contiguous() and wts.shape == (T, top) and wts.is_cuda, "wts")
+    if shared is not None:
+        _rows(shared, "shared", N, h.dtype)
+        _check(shared.shape[0] == T, "shared rows")
+    out = torch.empty(T, N, dtype=torch.float32, device=h.device)
+    if T == 0:
+        return out
+    P = T * top
+    maxt = -(-P // 64) + min(E, P)
+    _check(maxt <= 65535, "too many (token, expert) pairs in one step")
+    dev = h.device
+    meta = torch.empty(1 + (E + 1) + 2 * maxt, dtype=torch.int32, device=dev)
+    order = torch.empty(P, dtype=torch.int32, device=dev)
+    place = torch.empty(P, dtype=torch.int32, device=dev)
+    act = torch.empty(P, F, dtype=h.dtype, device=dev)
+    y = torch.empty(P, N, dtype=torch.float32, device=dev)
+    L = lib()
+    st = _stream()
+    L.moe_group(idx.data_ptr(), P, E, maxt, meta.data_ptr(), order.data_ptr(), place.data_ptr(), st)
+    L.moe_gate_up(h.data_ptr(), h.stride(0), gate.data_ptr(), up.data_ptr(), meta.data_ptr(), order.data_ptr(),
+                  act.data_ptr(), E, maxt, top, F, K, float(limit), float(alpha), dt, st)
+    L.moe_down(act.data_ptr(), down.data_ptr(), meta.data_ptr(), y.data_ptr(), E, maxt, N, F, dt, st)
+    L.moe_combine(y.data_ptr(), place.data_ptr(), wts.data_ptr(), _ptr(shared),
+                  shared.stride(0) if shared is not None else 0, out.data_ptr(), T, N, top, dt, st)
+    return out

@@ -446,3 +446,123 @@ def cross_entropy(logits: torch.Tensor, labels: torch.Tensor) -> torch.Tensor:
 
 def softmax_scale(D: int) -> float:
     return 1.0 / math.sqrt(D)
+
+
+# ------------------------------------------------------------------- fp32 residual stream / latent attention / MoE
+# CPU definitions of the kernels in csrc/resid32.hip, gemm_any.hip, attention_latent.hip and moe.hip: fp32 math,
+# results rounded to the storage type at the same places as on the GPU.
+def embed_scaled(ids: torch.Tensor, table: torch.Tensor, scale: float) -> torch.Tensor:
+    """fp32 rows table[ids] * scale."""
+    return table[ids.clamp(0, table.shape[0] - 1)].float() * scale
+
+
+def resid_add_norm(x: torch.Tensor, a, b, w, woff: float, eps: float, out_dtype, want_y: bool = True):
+    """x (fp32, in place) += (a + b) for the addends given; returns rms_norm(x) * (woff + w) in ``out_dtype``
+    (None when ``want_y`` is false)."""
+    if a is not None or b is not None:
+        d = a.float() if a is not None else None
+        if b is not None:
+            d = b.float() if d is None else d + b.float()
+        x.add_(d)
+    if not want_y:
+        return None
+    y = x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps) * (woff + w.float())
+    return y.to(out_dtype)
+
+
+def linear_f(x: torch.Tensor, w: torch.Tensor, out_dtype) -> torch.Tensor:
+    """x [M, K] . w [N, K]^T with fp32 accumulation -> [M, N] in ``out_dtype``."""
+    return (x.float() @ w.float().t()).to(out_dtype)
+
+
+def head_absorb(q: torch.Tensor, uk: torch.Tensor, H: int, dim: int) -> torch.Tensor:
+    """qa[t, h, :] = sum_d q[t, h * dim + d] * uk[h * dim + d, :] -> fp32 [T, H, R]."""
+    T = q.shape[0]
+    return torch.einsum("thd,hdr->thr", q[:, : H * dim].float().view(T, H, dim), uk.float().view(H, dim, -1))
+
+
+def head_expand(o: torch.Tensor, uv: torch.Tensor, out_dtype) -> torch.Tensor:
+    """y[t, h * vd + v] = sum_r o[t, h, r] * uv[h * vd + v, r] -> [T, H * vd] in ``out_dtype``."""
+    T, H, R = o.shape
+    return torch.einsum("thr,hvr->thv", o.float(), uv.float().view(H, -1, R)).reshape(T, -1).to(out_dtype)
+
+
+def latent_norm_cache(src: torch.Tensor, off: int, R: int, w: torch.Tensor, eps: float, cache: torch.Tensor,
+                      slots: torch.Tensor) -> None:
+    """cache[slot[t]] = rms_norm(src[t, off : off + R]) * w (slots < 0 are skipped); cache is [blocks, bs, R]."""
+    c = src[:, off:off + R].float()
+    c = c * torch.rsqrt(c.pow(2).mean(-1, keepdim=True) + eps) * w.float()
+    valid = slots >= 0
+    cache.view(-1, R)[slots[valid]] = c[valid].to(cache.dtype)
+
+
+def latent_attn(qa: torch.Tensor, cache: torch.Tensor, block_tables, cu_q, ctx_lens, window: int,
+                scale: float) -> torch.Tensor:
+    """Multi-query attention whose keys and values are the cached latent rows (csrc/attention_latent.hip):
+    qa fp32 [T, H, R]; sequence b's rows cu_q[b]:cu_q[b+1] sit at positions ctx_lens[b] - qlen .. ctx_lens[b] - 1
+    and see the positions j with 0 <= i - j (< window when window > 0). Returns fp32 [T, H, R]."""
+    T, H, R = qa.shape
+    bs = cache.shape[1]
+    out = torch.zeros(T, H, R, dtype=torch.float32, device=qa.device)
+    cu = [int(c) for c in cu_q.tolist()]
+    for b in range(len(cu) - 1):
+        a, e = cu[b], cu[b + 1]
+        ctx = int(ctx_lens[b])
+        if e == a or ctx <= 0:
+            continue
+        p0 = ctx - (e - a)
+        nblk = -(-ctx // bs)
+        c = cache[block_tables[b, :nblk].long()].reshape(nblk * bs, R)[:ctx].float()
+        s = torch.einsum("thr,jr->htj", qa[a:e].float() * scale, c)
+        i = torch.arange(p0, ctx, device=qa.device)[:, None]
+        j = torch.arange(ctx, device=qa.device)[None, :]
+        vis = (i - j >= 0)
+        if window > 0:
+            vis &= (i - j < window)
+        s = s.masked_fill(~vis, float("-inf"))
+        out[a:e] = torch.einsum("htj,jr->thr", torch.softmax(s, -1), c)
+    return out
+
+
+def glu_clamped(g: torch.Tensor, u: torch.Tensor, limit: float, alpha: float) -> torch.Tensor:
+    g = g.clamp(max=limit)
+    u = u.clamp(-limit, limit)
+    return g * torch.sigmoid(alpha * g) * (u + 1)
+
+
+def glu_clamp(gu: torch.Tensor, F_: int, limit: float, alpha: float) -> torch.Tensor:
+    """[T, 2F] gate | up halves -> [T, F]."""
+    return glu_clamped(gu[:, :F_].float(), gu[:, F_:2 * F_].float(), limit, alpha).to(gu.dtype)
+
+
+def moe_route(z: torch.Tensor, corr: Optional[torch.Tensor], top: int):
+    """fp32 router logits [T, E] -> (idx int32 [T, top], weights fp32 [T, top]): scores sigmoid(z), the ``top``
+    largest of score + corr chosen (ties: lower index), weights = chosen scores / (their sum + 1e-20)."""
+    s = torch.sigmoid(z.float())
+    ch = s if corr is None else s + corr.float()
+    # descending by value, ascending by index among equals
+    order = torch.argsort(ch, dim=-1, descending=True, stable=True)
+    idx = order[:, :top]
+    w = torch.gather(s, 1, idx)
+    w = w / (w.sum(-1, keepdim=True) + 1e-20)
+    return idx.to(torch.int32), w
+
+
+def moe_experts(h: torch.Tensor, idx: torch.Tensor, wts: torch.Tensor, gate: torch.Tensor, up: torch.Tensor,
+                down: torch.Tensor, limit: float, alpha: float, shared: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """sum_j wts[t, j] * down_e(glu(gate_e h, up_e h)) (+ shared) with e = idx[t, j] -> fp32 [T, N]. Stacked expert
+    weights gate / up [E, F, K], down [E, N, F]; the activation is rounded to the storage type between the
+    products, as the grouped GEMMs do."""
+    T = h.shape[0]
+    N = down.shape[1]
+    out = torch.zeros(T, N, dtype=torch.float32, device=h.device)
+    hf = h.float()
+    for j in range(idx.shape[1]):
+        for e in idx[:, j].unique().tolist():
+            rows = torch.nonzero(idx[:, j] == e).flatten()
+            x = hf[rows]
+            a = glu_clamped(x @ gate[e].float().t(), x @ up[e].float().t(), limit, alpha).to(h.dtype).float()
+            out[rows] += wts[rows, j:j + 1] * (a @ down[e].float().t())
+    if shared is not None:
+        out += shared.float()
+    return out
