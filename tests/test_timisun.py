@@ -80,13 +80,22 @@ class Case:
                          autotune=False, **kw)
 
     def ref(self, tokens):
+        """Oracle logits [T, V]; in bf16 runs the rows where some router's choice is a close call (the bf16 rounding
+        of its input may pick the other expert, which is no fault) are NaN and skipped by close()."""
         key = tuple(tokens)
         if key not in self._ref:
-            self._ref[key] = oracle.forward(self.cfg, self.sd, list(tokens))[0].float()
+            margins = []
+            lg = oracle.forward(self.cfg, self.sd, list(tokens), margins)[0].float()
+            if self.dtype != "float32" and margins:
+                lg[torch.stack(margins).min(0).values < 0.005] = float("nan")
+            self._ref[key] = lg
         return self._ref[key]
 
     def close(self, got, want, what=""):
         got, want = got.float().cpu(), want.float()
+        keep = ~torch.isnan(want).any(-1)
+        assert int(keep.sum()) >= 0.5 * len(keep), "too many close calls for a meaningful comparison"
+        got, want = got[keep], want[keep]
         d = (got - want) - (got - want).mean(-1, keepdim=True)
         err = d.pow(2).mean(-1).sqrt() / want.std(-1).clamp_min(1e-3)
         tol = 2e-4 if self.dtype == "float32" else 6e-2

@@ -61,6 +61,15 @@ def route(h, w_router, correction, top):
     return chosen, w / (w.sum(-1, keepdim=True) + 1e-20)
 
 
+def route_margin(h, w_router, correction, top):
+    """How far the last chosen expert's choice score lies above the first one left out, per token (inf when every
+    expert is chosen): rows with a tiny margin are close calls that rounding may decide either way."""
+    ch = torch.sort(torch.sigmoid(h @ w_router.T) + correction, dim=-1, descending=True).values
+    if top >= ch.shape[1]:
+        return torch.full((h.shape[0],), math.inf, dtype=h.dtype)
+    return ch[:, top - 1] - ch[:, top]
+
+
 def moe(h, sd, p, spec):
     chosen, w = route(h, sd[p + "router"], sd[p + "correction"], spec["router"]["top"])
     out = torch.zeros_like(h)
@@ -75,8 +84,9 @@ def moe(h, sd, p, spec):
     return out
 
 
-def forward(cfg, sd, tokens):
-    """cfg: the config.json dict; sd: name -> tensor. Returns (logits [T, V], [residual after each layer])."""
+def forward(cfg, sd, tokens, margins=None):
+    """cfg: the config.json dict; sd: name -> tensor. Returns (logits [T, V], [residual after each layer]); a list
+    given as ``margins`` receives every feed-forward's route_margin."""
     sd = {k: v.double() for k, v in sd.items()}
     eps = cfg["norm"]["eps"]
     x = sd["embed"][torch.tensor(tokens)] * cfg["embedding"]["scale"]
@@ -93,6 +103,8 @@ def forward(cfg, sd, tokens):
         a = latent_attention(h, c, sd[p + "mix.q"], sd[p + "mix.uk"], sd[p + "mix.uv"], sd[p + "mix.o"], m["heads"],
                              m["dim"], m["vdim"], m["scale"], window)
         f = moe(h, sd, p + "mlp.", L["mlp"]) if L.get("mlp") else torch.zeros_like(x)
+        if margins is not None and L.get("mlp"):
+            margins.append(route_margin(h, sd[p + "mlp.router"], sd[p + "mlp.correction"], L["mlp"]["router"]["top"]))
         x = x + (a + f)
         stream.append(x.clone())
     return norm_around_zero(x, sd["final.norm"], eps) @ sd["embed"].T, stream
