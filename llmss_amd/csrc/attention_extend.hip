@@ -17,6 +17,11 @@
 //   S^T[key][slot] = K . Q^T   (A = K rows via ds_read_b128, B = Q^T fragments in registers)
 //   O^T[d][slot]  += V^T . P^T (A = V^T via ds_read_tr16_b64, B = P^T straight from S^T)
 // so each lane owns one slot's softmax row.
+//
+// Sliding window (window > 0): query position p attends keys (p - window, p] only; the key loop starts at the tile
+// holding the first row's oldest visible key, and tiles wholly before a wave's window are skipped.
+// SAME: keys and values are one tensor (latent attention, where both are the cached latent row and nkv = 1): the
+// tile is loaded and staged once and serves both products.
 #include "common.h"
 
 constexpr float kLog2eX = 1.4426950408889634f;
@@ -27,16 +32,18 @@ constexpr float kLog2eX = 1.4426950408889634f;
 // absmax / 448 scale and clamped conversion) for the W8A8 o-projection that consumes them, which then skips its own
 // quantisation launch. Only when a workgroup holds every head of its rows: one kv head (nkv = 1) whose whole query
 // group fits the slots of a wave (GE = G, a power of two <= 16) - Llama-2-70B at TP=8 (8 query heads per rank).
-template <int D, bool KV8>
+template <int D, bool KV8, bool SAME = false>
 __global__ __launch_bounds__(256) void attn_extend_kernel(
     const bf16_t* __restrict__ q, int64_t q_stride, const void* __restrict__ kcv, const void* __restrict__ vcv,
     const int* __restrict__ block_tables, int max_blocks, const int* __restrict__ cu_q, const int* __restrict__ ctx_lens,
     bf16_t* __restrict__ out, int64_t out_stride, int nh, int nkv, int GE, int bs, float scale_log2,
-    unsigned char* __restrict__ q8, float* __restrict__ s8) {
+    unsigned char* __restrict__ q8, float* __restrict__ s8, int window) {
+  static_assert(!(SAME && KV8), "a shared key/value tile is staged from bf16 rows");
   constexpr int BKV = 64;
   constexpr int LD = D + 16;  // padded LDS row (elements): conflict-free b128 rows and tr_b16 columns
   __shared__ __attribute__((aligned(16))) bf16_t Ks[BKV * LD];
-  __shared__ __attribute__((aligned(16))) bf16_t Vs[BKV * LD];
+  __shared__ __attribute__((aligned(16))) bf16_t Vs_[SAME ? 8 : BKV * LD];
+  bf16_t* const Vs = SAME ? Ks : Vs_;
 
   const int G = nh / nkv;
   const int rows_per_wg = 64 / GE;
@@ -71,6 +78,9 @@ __global__ __launch_bounds__(256) void attn_extend_kernel(
   const int kv_end = p0 + r_last + 1;
   // this wave's slots: rows r0 + (16w)/GE .. r0 + (16w+15)/GE
   const int wave_qhi = p0 + min(qlen - 1, r0 + (16 * w + 15) / GE);
+  // first key any row of the workgroup / of this wave may see (tile-aligned start of the key loop)
+  const int kv_begin = window > 0 ? max(0, p0 + r0 - window + 1) / BKV * BKV : 0;
+  const int wave_klo = window > 0 ? p0 + min(qlen - 1, r0 + (16 * w) / GE) - window + 1 : 0;
   const int* bt = block_tables + (int64_t)b * max_blocks;
   constexpr int CH = D / 8;
   constexpr int RB = KV8 ? D + 16 : D;         // cache row (elements of the cache dtype)
@@ -111,7 +121,7 @@ __global__ __launch_bounds__(256) void attn_extend_kernel(
         vsr[j] = *reinterpret_cast<const float*>(vc8 + rowoff + D);
       } else {
         kr[j] = *reinterpret_cast<const u16x8*>(kc + rowoff + ch * 8);
-        vr[j] = *reinterpret_cast<const u16x8*>(vc + rowoff + ch * 8);
+        if constexpr (!SAME) vr[j] = *reinterpret_cast<const u16x8*>(vc + rowoff + ch * 8);
       }
     }
   };
@@ -135,7 +145,7 @@ __global__ __launch_bounds__(256) void attn_extend_kernel(
         *reinterpret_cast<u16x8*>(&Vs[r * LD + ch * 8]) = vb;
       } else {
         *reinterpret_cast<u16x8*>(&Ks[r * LD + ch * 8]) = kr[j];
-        *reinterpret_cast<u16x8*>(&Vs[r * LD + ch * 8]) = vr[j];
+        if constexpr (!SAME) *reinterpret_cast<u16x8*>(&Vs[r * LD + ch * 8]) = vr[j];
       }
     }
   };
@@ -167,14 +177,15 @@ __global__ __launch_bounds__(256) void attn_extend_kernel(
         *reinterpret_cast<u16x8*>(&Vs[r * LD + ch * 8]) = vb;
       } else {
         *reinterpret_cast<u16x8*>(&Ks[r * LD + ch * 8]) = *reinterpret_cast<const u16x8*>(kc + rowoff + ch * 8);
-        *reinterpret_cast<u16x8*>(&Vs[r * LD + ch * 8]) = *reinterpret_cast<const u16x8*>(vc + rowoff + ch * 8);
+        if constexpr (!SAME)
+          *reinterpret_cast<u16x8*>(&Vs[r * LD + ch * 8]) = *reinterpret_cast<const u16x8*>(vc + rowoff + ch * 8);
       }
     }
   };
   if constexpr (PIPE) {
-    if (kv_end > 0) load_tile(0);
+    if (kv_end > kv_begin) load_tile(kv_begin);
   }
-  for (int kv0 = 0; kv0 < kv_end; kv0 += BKV) {
+  for (int kv0 = kv_begin; kv0 < kv_end; kv0 += BKV) {
     __syncthreads();  // every wave is done reading the previous tile
     if constexpr (PIPE) store_tile();
     else stage_direct(kv0);
@@ -183,6 +194,7 @@ __global__ __launch_bounds__(256) void attn_extend_kernel(
       if (kv0 + BKV < kv_end) load_tile(kv0 + BKV);
     }
     if (kv0 > wave_qhi) continue;  // whole tile in this wave's causal future (barriers stay uniform)
+    if (kv0 + BKV <= wave_klo) continue;  // whole tile older than this wave's windows
 
     f32x4 s[4];
 #pragma unroll
@@ -202,7 +214,7 @@ __global__ __launch_bounds__(256) void attn_extend_kernel(
       for (int i = 0; i < 4; ++i) {
         const int key = kv0 + kt * 16 + 4 * g + i;
         float v = s[kt][i] * scale_log2;
-        v = (key <= qpos && key < kv_end) ? v : -1.0e30f;
+        v = (key <= qpos && key < kv_end && (window <= 0 || key > qpos - window)) ? v : -1.0e30f;
         s[kt][i] = v;
         mx = fmaxf(mx, v);
       }
@@ -216,7 +228,8 @@ __global__ __launch_bounds__(256) void attn_extend_kernel(
     for (int kt = 0; kt < 4; ++kt)
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        const float p = exp2f(s[kt][i] - mx);
+        // a masked key adds nothing, also while a slot has seen no visible key yet (mx still at its floor)
+        const float p = s[kt][i] > -1.0e29f ? exp2f(s[kt][i] - mx) : 0.f;
         const bf16_t pb = f2bf(p);
         ps += bf2f(pb);
         pf[kt >> 1][(kt & 1) * 4 + i] = (short)pb;
@@ -289,7 +302,7 @@ static int extend_group(int G) {
 void launch_attn_extend(const void* q, int64_t q_stride, const void* k_cache, const void* v_cache,
                         const void* block_tables, int max_blocks, const void* cu_q, const void* ctx_lens, void* out,
                         int64_t out_stride, int B, int max_qlen, int nh, int nkv, int D, int bs, float scale,
-                        hipStream_t st, bool kv8, void* q8v, void* s8v) {
+                        hipStream_t st, bool kv8, void* q8v, void* s8v, int window) {
   if (nh % nkv) throw std::runtime_error("attn_extend: nh must be a multiple of nkv");
   if (B == 0 || max_qlen == 0) return;
   const int G = nh / nkv, GE = extend_group(G);
@@ -308,14 +321,19 @@ void launch_attn_extend(const void* q, int64_t q_stride, const void* k_cache, co
   auto CL = (const int*)ctx_lens;
   auto O = (bf16_t*)out;
   const float sl = scale * kLog2eX;
+  const bool same = !kv8 && k_cache == v_cache && nkv == 1;
+  if (window < 0) throw std::runtime_error("attn_extend: negative window");
 #define LX(D_)                                                                                                   \
   do {                                                                                                           \
     if (kv8)                                                                                                     \
       attn_extend_kernel<D_, true><<<grid, 256, 0, st>>>(Q, q_stride, K, V, BT, max_blocks, CU, CL, O, out_stride, nh, \
-                                                         nkv, GE, bs, sl, Q8, S8);                               \
+                                                         nkv, GE, bs, sl, Q8, S8, window);                       \
+    else if (same)                                                                                               \
+      attn_extend_kernel<D_, false, true><<<grid, 256, 0, st>>>(Q, q_stride, K, V, BT, max_blocks, CU, CL, O,          \
+                                                                out_stride, nh, nkv, GE, bs, sl, Q8, S8, window); \
     else                                                                                                         \
       attn_extend_kernel<D_, false><<<grid, 256, 0, st>>>(Q, q_stride, K, V, BT, max_blocks, CU, CL, O, out_stride,   \
-                                                          nh, nkv, GE, bs, sl, Q8, S8);                          \
+                                                          nh, nkv, GE, bs, sl, Q8, S8, window);                  \
   } while (0)
   switch (D) {
     case 64: LX(64); break;

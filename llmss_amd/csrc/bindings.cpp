@@ -38,7 +38,7 @@ void launch_ce_loss(const void* logits, int64_t ld, bool fp32, const void* label
 void launch_attn_extend(const void* q, int64_t q_stride, const void* k_cache, const void* v_cache,
                         const void* block_tables, int max_blocks, const void* cu_q, const void* ctx_lens, void* out,
                         int64_t out_stride, int B, int max_qlen, int nh, int nkv, int D, int bs, float scale,
-                        hipStream_t st, bool kv8, void* q8, void* s8);
+                        hipStream_t st, bool kv8, void* q8, void* s8, int window);
 int launch_gemm_qkv_args(const void* x, int64_t ldx, const void* w, int64_t ldw, const void* bias, void* y, int64_t ldy,
                          int M, int N, int K, void* workspace, int64_t ws_bytes, int nt_hint, int split_hint,
                          const void* pos, const void* cos_t, const void* sin_t, void* kc, void* vc, const void* slot,
@@ -80,6 +80,13 @@ void launch_resid_add_norm(void* x, const void* a, int64_t lda, const void* b, i
 void launch_gemm_any(const void* A, const void* B, void* C, int M, int N, int K, int batch, int64_t sAb, int64_t sAm,
                      int64_t sBb, int64_t sBn, int64_t sBk, int64_t sCb, int64_t sCm, int da, int db, int dc,
                      hipStream_t st);
+void launch_gemm_tile(const void* A, const void* B, void* C, int M, int N, int K, int batch, int64_t sAb, int64_t sAm,
+                      int64_t sBb, int64_t sBn, int64_t sCb, int64_t sCm, int dc, hipStream_t st);
+void launch_moe_gate_up_tile(const void* h, int64_t ldh, const void* wg, const void* wu, const void* meta,
+                             const void* order, void* act, int E, int maxt, int top, int F, int K, float limit,
+                             float alpha, hipStream_t st);
+void launch_moe_down_tile(const void* act, const void* wd, const void* meta, void* y, int E, int maxt, int N, int F,
+                          hipStream_t st);
 void launch_latent_norm_cache(const void* src, int64_t ld, int off, const void* w, float eps, void* cache,
                               const void* slots, int T_, int R, int dt, hipStream_t st);
 void launch_latent_attn(const void* qa, int64_t ldq, const void* cache, const void* bt, int maxb, const void* cu_q,
@@ -151,14 +158,14 @@ PYBIND11_MODULE(_C, m) {
   });
   m.def("attn_extend", [](uintptr_t q, int64_t qs, uintptr_t kc, uintptr_t vc, uintptr_t bt, int maxb, uintptr_t cu,
                           uintptr_t cl, uintptr_t out, int64_t os, int B, int maxq, int nh, int nkv, int D, int bs,
-                          float scale, uintptr_t st, bool kv8, uintptr_t q8, uintptr_t s8) {
+                          float scale, uintptr_t st, bool kv8, uintptr_t q8, uintptr_t s8, int window) {
     launch_attn_extend(CP(q), qs, CP(kc), CP(vc), CP(bt), maxb, CP(cu), CP(cl), P(out), os, B, maxq, nh, nkv, D, bs,
-                       scale, S(st), kv8, P(q8), P(s8));
+                       scale, S(st), kv8, P(q8), P(s8), window);
   }, pybind11::arg("q"), pybind11::arg("qs"), pybind11::arg("kc"), pybind11::arg("vc"), pybind11::arg("bt"),
      pybind11::arg("maxb"), pybind11::arg("cu"), pybind11::arg("cl"), pybind11::arg("out"), pybind11::arg("os"),
      pybind11::arg("B"), pybind11::arg("maxq"), pybind11::arg("nh"), pybind11::arg("nkv"), pybind11::arg("D"),
      pybind11::arg("bs"), pybind11::arg("scale"), pybind11::arg("st"), pybind11::arg("kv8"), pybind11::arg("q8") = 0,
-     pybind11::arg("s8") = 0);
+     pybind11::arg("s8") = 0, pybind11::arg("window") = 0);
   m.def("gemm", [](uintptr_t x, int64_t ldx, uintptr_t w, int64_t ldw, bool fp8, uintptr_t ws, uintptr_t bias,
                    uintptr_t y, int64_t ldy, int M, int N, int K, int act, bool glu, uintptr_t work, int64_t wbytes,
                    int nt_hint, int split_hint, bool partial_out, uintptr_t st) {
@@ -243,6 +250,18 @@ PYBIND11_MODULE(_C, m) {
                        uintptr_t st) {
     launch_gemm_any(CP(A), CP(B), P(C), M, N, K, batch, sAb, sAm, sBb, sBn, sBk, sCb, sCm, da, db, dc, S(st));
   });
+  m.def("gemm_tile", [](uintptr_t A, uintptr_t B, uintptr_t C, int M, int N, int K, int batch, int64_t sAb, int64_t sAm,
+                        int64_t sBb, int64_t sBn, int64_t sCb, int64_t sCm, int dc, uintptr_t st) {
+    launch_gemm_tile(CP(A), CP(B), P(C), M, N, K, batch, sAb, sAm, sBb, sBn, sCb, sCm, dc, S(st));
+  });
+  m.def("moe_gate_up_tile", [](uintptr_t h, int64_t ldh, uintptr_t wg, uintptr_t wu, uintptr_t meta, uintptr_t order,
+                               uintptr_t act, int E, int maxt, int top, int F, int K, float limit, float alpha,
+                               uintptr_t st) {
+    launch_moe_gate_up_tile(CP(h), ldh, CP(wg), CP(wu), CP(meta), CP(order), P(act), E, maxt, top, F, K, limit, alpha,
+                            S(st));
+  });
+  m.def("moe_down_tile", [](uintptr_t act, uintptr_t wd, uintptr_t meta, uintptr_t y, int E, int maxt, int N, int F,
+                            uintptr_t st) { launch_moe_down_tile(CP(act), CP(wd), CP(meta), P(y), E, maxt, N, F, S(st)); });
   m.def("latent_norm_cache", [](uintptr_t src, int64_t ld, int off, uintptr_t w, float eps, uintptr_t cache,
                                 uintptr_t slots, int T, int R, int dt, uintptr_t st) {
     launch_latent_norm_cache(CP(src), ld, off, CP(w), eps, P(cache), CP(slots), T, R, dt, S(st));

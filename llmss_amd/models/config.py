@@ -121,6 +121,16 @@ class ModelConfig:
 
     def num_params(self) -> int:
         h, f, v = self.hidden_size, self.intermediate_size, self.vocab_size
+        if self.layer_specs:
+            n = v * h + h
+            for s in self.layer_specs:
+                m = s.mixer
+                n += h + m.heads * m.dim * h + (m.kv_rank * (h + 1) if m.kv_from is None else 0)
+                n += m.heads * (m.dim + m.vdim) * m.kv_rank + h * m.heads * m.vdim
+                if s.mlp is not None:
+                    n += s.mlp.experts * (h + 1 + 3 * h * s.mlp.expert.ff)
+                    n += 3 * h * s.mlp.shared.ff if s.mlp.shared else 0
+            return n
         attn = h * (self.q_size + 2 * self.kv_size) + self.q_size * h
         mlp = (3 if self.gated_mlp else 2) * h * f
         per_layer = attn + mlp + 4 * h

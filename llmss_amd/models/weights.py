@@ -537,17 +537,18 @@ def shard_cache_path(root: str, model_dir: str, files: List[str], tp: int, rank:
 class LatentAttnWeights:
     """Latent attention: ``qc`` [heads * dim (+ kv_rank), H] is the query projection followed, in a layer that
     projects its own latent rows (``own_kv``), by the latent down-projection - one GEMM for both; ``kv_norm``
-    [kv_rank] the latent's plain RMS-norm weight; ``uk`` [heads * dim, kv_rank] and ``uv`` [heads * vdim, kv_rank]
-    the per-head key / value up-projections; ``o`` [H, heads * vdim]."""
+    [kv_rank] the latent's plain RMS-norm weight; ``uk_t`` [heads, kv_rank, dim] the key up-projection, per head
+    transposed (the absorbed query is q_h . uk_h: dim is then the contiguous contraction index); ``uv``
+    [heads * vdim, kv_rank] the value up-projection; ``o`` [H, heads * vdim]."""
     qc: torch.Tensor
     own_kv: bool
     kv_norm: Optional[torch.Tensor]
-    uk: torch.Tensor
+    uk_t: torch.Tensor
     uv: torch.Tensor
     o: torch.Tensor
 
     def tensors(self):
-        return [t for t in (self.qc, self.kv_norm, self.uk, self.uv, self.o) if t is not None]
+        return [t for t in (self.qc, self.kv_norm, self.uk_t, self.uv, self.o) if t is not None]
 
 
 @dataclass
@@ -587,6 +588,12 @@ def _tied_head(cfg: ModelConfig, wte: torch.Tensor, device, dtype):
     return table[:cfg.vocab_size], Linear(table)
 
 
+def _heads_t(uk: torch.Tensor, heads: int, dim: int, rank: int, layer: int) -> torch.Tensor:
+    if tuple(uk.shape) != (heads * dim, rank):
+        raise ValueError(f"layer {layer}: uk has shape {tuple(uk.shape)}, the config says {(heads * dim, rank)}")
+    return uk.view(heads, dim, rank).transpose(1, 2).contiguous()
+
+
 def _timisun_finish(cfg: ModelConfig, get, device, dtype) -> ModelWeights:
     """``get(name)`` returns the checkpoint tensor of that name (CPU); tensor names as in the checkpoint:
     ``embed``, ``final.norm``, ``l<i>.norm1``, ``l<i>.mix.{q,dkv,dkv.norm,uk,uv,o}``,
@@ -603,9 +610,10 @@ def _timisun_finish(cfg: ModelConfig, get, device, dtype) -> ModelWeights:
         mix = LatentAttnWeights(
             qc=dev(torch.cat([q, get(p + "mix.dkv")], 0) if own else q), own_kv=own,
             kv_norm=dev(get(p + "mix.dkv.norm")) if own else None,
-            uk=dev(get(p + "mix.uk")), uv=dev(get(p + "mix.uv")), o=dev(get(p + "mix.o")))
+            uk_t=dev(_heads_t(get(p + "mix.uk"), mx.heads, mx.dim, mx.kv_rank, i)), uv=dev(get(p + "mix.uv")),
+            o=dev(get(p + "mix.o")))
         want = {"qc": (mx.heads * mx.dim + (mx.kv_rank if own else 0), cfg.hidden_size),
-                "uk": (mx.heads * mx.dim, mx.kv_rank), "uv": (mx.heads * mx.vdim, mx.kv_rank),
+                "uk_t": (mx.heads, mx.kv_rank, mx.dim), "uv": (mx.heads * mx.vdim, mx.kv_rank),
                 "o": (cfg.hidden_size, mx.heads * mx.vdim)}
         for nm, shp in want.items():
             if tuple(getattr(mix, nm).shape) != shp:

@@ -73,13 +73,13 @@ def attn_decode(q, k_cache, v_cache, block_tables, ctx_lens, nh, nkv, D, scale, 
 
 
 def attn_extend(q, k_cache, v_cache, block_tables, cu_q, ctx_lens, max_qlen, nh, nkv, D, scale, out=None,
-                fp8_out=False):
+                fp8_out=False, window=0):
     """Chunked-prefill attention over the paged cache (the chunk's K/V already written). ``fp8_out``: the GPU
     kernel also writes the per-token fp8 twin for a W8A8 consumer (ops.hip.attn_extend); ignored on the CPU."""
     if q.is_cuda:
         return _hip().attn_extend(q, k_cache, v_cache, block_tables, cu_q, ctx_lens, max_qlen, nh, nkv, D, scale,
-                                  out=out, fp8_out=fp8_out)
-    return _into(ref.attn_extend(q, k_cache, v_cache, block_tables, cu_q, ctx_lens, nh, nkv, D, scale), out)
+                                  out=out, fp8_out=fp8_out, window=window)
+    return _into(ref.attn_extend(q, k_cache, v_cache, block_tables, cu_q, ctx_lens, nh, nkv, D, scale, window), out)
 
 
 def linear(x, w, bias=None, act="none", glu=False, w_scale: Optional[torch.Tensor] = None, partial_ok=False):
@@ -169,6 +169,7 @@ head_absorb = _route("head_absorb")
 head_expand = _route("head_expand")
 latent_norm_cache = _route("latent_norm_cache")
 latent_attn = _route("latent_attn")
+latent_qa_dtype = _route("latent_qa_dtype")
 glu_clamp = _route("glu_clamp")
 moe_route = _route("moe_route")
 moe_experts = _route("moe_experts")

@@ -194,10 +194,11 @@ def extend_fp8_twin_ok(nh: int, nkv: int) -> bool:
 
 
 def attn_extend(q, k_cache, v_cache, block_tables, cu_q, ctx_lens, max_qlen, nh, nkv, D, scale, out=None,
-                fp8_out=False):
+                fp8_out=False, window=0):
     """Chunked-prefill attention: q rows [T, >= nh*D] (query heads first, as in the QKV output) of B
     sequences (``cu_q`` [B+1] int32), each attending its whole paged context ``ctx_lens`` [B] int32 (the
-    chunk's own K/V already written to the cache) causally. ``fp8_out`` (only where extend_fp8_twin_ok):
+    chunk's own K/V already written to the cache) causally; ``window`` > 0 limits a position to itself and the
+    ``window - 1`` positions before it. ``fp8_out`` (only where extend_fp8_twin_ok):
     also write the output's per-token fp8 twin for the W8A8 o-projection, which then skips its quantisation
     launch."""
     T = q.shape[0]
@@ -221,7 +222,7 @@ def attn_extend(q, k_cache, v_cache, block_tables, cu_q, ctx_lens, max_qlen, nh,
         q8, s8 = _fp8_twin(y)
     lib().attn_extend(q.data_ptr(), q.stride(0), k_cache.data_ptr(), v_cache.data_ptr(), block_tables.data_ptr(),
                       block_tables.shape[1], cu_q.data_ptr(), ctx_lens.data_ptr(), y.data_ptr(), y.stride(0), B,
-                      int(max_qlen), nh, nkv, D, bs, float(scale), _stream(), kv8, _ptr(q8), _ptr(s8))
+                      int(max_qlen), nh, nkv, D, bs, float(scale), _stream(), kv8, _ptr(q8), _ptr(s8), int(window))
     return y
 
 
@@ -829,8 +830,13 @@ def resid_add_norm(x, a, b, w, woff, eps, out_dtype, want_y=True):
 
 
 def gemm_any(A, B, C, M, N, K, batch, sAb, sAm, sBb, sBn, sBk, sCb, sCm):
-    """C[b][m][n] = sum_k A[b][m][k] B[b][n][k] over element strides (csrc/gemm_any.hip); the caller has checked that
-    every index stays inside its tensor."""
+    """C[b][m][n] = sum_k A[b][m][k] B[b][n][k] over element strides; the caller has checked that every index stays
+    inside its tensor. bf16 operands with k contiguous run on the matrix cores (csrc/gemm_tile.hip), everything else
+    (fp32 storage, k-major B) on the vector ALUs (csrc/gemm_any.hip)."""
+    if A.dtype == torch.bfloat16 and B.dtype == torch.bfloat16 and sBk == 1:
+        lib().gemm_tile(A.data_ptr(), B.data_ptr(), C.data_ptr(), int(M), int(N), int(K), int(batch), int(sAb),
+                        int(sAm), int(sBb), int(sBn), int(sCb), int(sCm), _dt(C, "C"), _stream())
+        return C
     lib().gemm_any(A.data_ptr(), B.data_ptr(), C.data_ptr(), int(M), int(N), int(K), int(batch), int(sAb), int(sAm),
                    int(sBb), int(sBn), int(sBk), int(sCb), int(sCm), _dt(A, "A"), _dt(B, "B"), _dt(C, "C"), _stream())
     return C
@@ -859,23 +865,22 @@ def linear_f(x, w, out_dtype):
     return gemm_any(x, w, y, M, N, K, 1, 0, x.stride(0), 0, K, 1, 0, N)
 
 
-def head_absorb(q, uk, H, dim):
+def head_absorb(q, uk_t, out_dtype=torch.float32):
+    H, R, dim = uk_t.shape
     T = q.shape[0]
-    R = uk.shape[1]
     _rows(q, "q")
     _check(q.shape[1] >= H * dim, "q too narrow")
-    _rows(uk, "uk")
-    _check(uk.is_contiguous() and uk.shape[0] == H * dim, "uk [H * dim, R]")
-    qa = torch.empty(T, H, R, dtype=torch.float32, device=q.device)
+    _check(uk_t.is_contiguous() and uk_t.dtype == q.dtype and uk_t.is_cuda, "uk_t [H, R, dim] in q's storage type")
+    qa = torch.empty(T, H, R, dtype=out_dtype, device=q.device)
     if T:
-        # batch = head: A(t, d) = q[t, h * dim + d]; B(r, d) = uk[h * dim + d, r]
-        gemm_any(q, uk, qa, T, R, dim, H, dim, q.stride(0), dim * R, 1, R, R, H * R)
+        # batch = head: A(t, d) = q[t, h * dim + d]; B(r, d) = uk_t[h, r, d]
+        gemm_any(q, uk_t, qa, T, R, dim, H, dim, q.stride(0), R * dim, dim, 1, R, H * R)
     return qa
 
 
 def head_expand(o, uv, out_dtype):
     T, H, R = o.shape
-    _check(o.is_contiguous() and o.dtype == torch.float32 and o.is_cuda, "o fp32 [T, H, R] contiguous")
+    _check(o.is_contiguous() and o.dtype in _DT and o.is_cuda, "o [T, H, R] contiguous")
     _rows(uv, "uv", R)
     _check(uv.is_contiguous() and uv.shape[0] % H == 0, "uv [H * vdim, R]")
     vd = uv.shape[0] // H
@@ -898,14 +903,34 @@ def latent_norm_cache(src, off, R, w, eps, cache, slots):
                             slots.data_ptr(), T, R, _dt(src, "src"), _stream())
 
 
-def latent_attn(qa, cache, block_tables, cu_q, ctx_lens, window, scale):
+LATENT_MFMA_RANKS = (64, 128, 256)  # latent ranks the MFMA extend kernel is built for (csrc/attention_extend.hip)
+
+
+def latent_qa_dtype(cache) -> torch.dtype:
+    """Storage type latent_attn wants its absorbed queries in: bf16 where the MFMA kernel runs, else fp32."""
+    if cache.is_cuda and cache.dtype == torch.bfloat16 and cache.shape[2] in LATENT_MFMA_RANKS:
+        return torch.bfloat16
+    return torch.float32
+
+
+def latent_attn(qa, cache, block_tables, cu_q, ctx_lens, window, scale, max_qlen=0):
+    """``qa`` [T, H, R]. bf16 queries over a bf16 cache of rank 64 / 128 / 256 run the MFMA extend kernel as
+    multi-query attention whose one key/value head is the latent row (keys = values = cache, bf16 output); anything
+    else runs the generic kernel (fp32 queries, fp32 output)."""
     T, H, R = qa.shape
-    _check(qa.is_contiguous() and qa.dtype == torch.float32 and qa.is_cuda, "qa fp32 [T, H, R] contiguous")
+    _check(qa.is_contiguous() and qa.is_cuda, "qa [T, H, R] contiguous")
     _check(cache.is_contiguous() and cache.dim() == 3 and cache.shape[2] == R, "latent cache [blocks, block_size, R]")
     B = cu_q.numel() - 1
     for t, nm in ((cu_q, "cu_q"), (ctx_lens, "ctx_lens"), (block_tables, "block_tables")):
         _check(t.dtype == torch.int32 and t.is_contiguous() and t.is_cuda, f"{nm} must be contiguous int32 cuda")
     _check(ctx_lens.numel() >= B and block_tables.dim() == 2 and block_tables.shape[0] >= B, "batch sizes")
+    if qa.dtype == torch.bfloat16:
+        _check(latent_qa_dtype(cache) == torch.bfloat16 and max_qlen > 0, "bf16 queries: MFMA ranks and max_qlen only")
+        kv = cache.view(cache.shape[0], 1, cache.shape[1], R)  # [blocks, one kv head, block_size, R]
+        out = attn_extend(qa.view(T, H * R), kv, kv, block_tables, cu_q, ctx_lens[:B], max_qlen, H, 1, R, scale,
+                          window=window)
+        return out.view(T, H, R)
+    _check(qa.dtype == torch.float32, "qa fp32")
     _check(R <= 512, "latent rank above 512")
     out = torch.empty(T, H, R, dtype=torch.float32, device=qa.device)
     lib().latent_attn(qa.data_ptr(), H * R, cache.data_ptr(), block_tables.data_ptr(), block_tables.shape[1],
@@ -967,9 +992,14 @@ def moe_experts(h, idx, wts, gate, up, down, limit, alpha, shared=None):
     L = lib()
     st = _stream()
     L.moe_group(idx.data_ptr(), P, E, maxt, meta.data_ptr(), order.data_ptr(), place.data_ptr(), st)
-    L.moe_gate_up(h.data_ptr(), h.stride(0), gate.data_ptr(), up.data_ptr(), meta.data_ptr(), order.data_ptr(),
-                  act.data_ptr(), E, maxt, top, F, K, float(limit), float(alpha), dt, st)
-    L.moe_down(act.data_ptr(), down.data_ptr(), meta.data_ptr(), y.data_ptr(), E, maxt, N, F, dt, st)
+    if h.dtype == torch.bfloat16:  # matrix cores (csrc/gemm_tile.hip)
+        L.moe_gate_up_tile(h.data_ptr(), h.stride(0), gate.data_ptr(), up.data_ptr(), meta.data_ptr(),
+                           order.data_ptr(), act.data_ptr(), E, maxt, top, F, K, float(limit), float(alpha), st)
+        L.moe_down_tile(act.data_ptr(), down.data_ptr(), meta.data_ptr(), y.data_ptr(), E, maxt, N, F, st)
+    else:
+        L.moe_gate_up(h.data_ptr(), h.stride(0), gate.data_ptr(), up.data_ptr(), meta.data_ptr(), order.data_ptr(),
+                      act.data_ptr(), E, maxt, top, F, K, float(limit), float(alpha), dt, st)
+        L.moe_down(act.data_ptr(), down.data_ptr(), meta.data_ptr(), y.data_ptr(), E, maxt, N, F, dt, st)
     L.moe_combine(y.data_ptr(), place.data_ptr(), wts.data_ptr(), _ptr(shared),
                   shared.stride(0) if shared is not None else 0, out.data_ptr(), T, N, top, dt, st)
     return out

@@ -208,7 +208,7 @@ def attn_decode(q: torch.Tensor, k_cache, v_cache, block_tables, ctx_lens, nh: i
 
 
 def attn_extend(q: torch.Tensor, k_cache, v_cache, block_tables, cu_q, ctx_lens, nh: int, nkv: int, D: int,
-                scale: float) -> torch.Tensor:
+                scale: float, window: int = 0) -> torch.Tensor:
     """Chunked prefill over the paged cache: sequence b's rows cu_q[b]:cu_q[b+1] sit at positions
     ctx_lens[b] - qlen ... ctx_lens[b] - 1 and attend every cached key up to their own position."""
     T = q.shape[0]
@@ -226,7 +226,8 @@ def attn_extend(q: torch.Tensor, k_cache, v_cache, block_tables, cu_q, ctx_lens,
         v = gather_kv(v_cache, block_tables[b], ctx).float().repeat_interleave(g, 0)
         s = torch.matmul(qq, k.transpose(1, 2)) * scale
         qpos = torch.arange(p0, ctx, device=q.device)[:, None]
-        s = s.masked_fill(torch.arange(ctx, device=q.device)[None, :] > qpos, float("-inf"))
+        kpos = torch.arange(ctx, device=q.device)[None, :]
+        s = s.masked_fill((kpos > qpos) | ((kpos <= qpos - window) if window > 0 else False), float("-inf"))
         out[a:e] = torch.matmul(torch.softmax(s, -1), v).transpose(0, 1).reshape(e - a, nh * D).to(q.dtype)
     return out
 
@@ -475,10 +476,16 @@ def linear_f(x: torch.Tensor, w: torch.Tensor, out_dtype) -> torch.Tensor:
     return (x.float() @ w.float().t()).to(out_dtype)
 
 
-def head_absorb(q: torch.Tensor, uk: torch.Tensor, H: int, dim: int) -> torch.Tensor:
-    """qa[t, h, :] = sum_d q[t, h * dim + d] * uk[h * dim + d, :] -> fp32 [T, H, R]."""
+def head_absorb(q: torch.Tensor, uk_t: torch.Tensor, out_dtype=torch.float32) -> torch.Tensor:
+    """qa[t, h, r] = sum_d q[t, h * dim + d] * uk_t[h, r, d] -> [T, H, R] (uk_t: the key up-projection, per head
+    transposed to [R, dim])."""
+    H, R, dim = uk_t.shape
     T = q.shape[0]
-    return torch.einsum("thd,hdr->thr", q[:, : H * dim].float().view(T, H, dim), uk.float().view(H, dim, -1))
+    return torch.einsum("thd,hrd->thr", q[:, : H * dim].float().view(T, H, dim), uk_t.float()).to(out_dtype)
+
+
+def latent_qa_dtype(cache) -> torch.dtype:
+    return torch.float32
 
 
 def head_expand(o: torch.Tensor, uv: torch.Tensor, out_dtype) -> torch.Tensor:
@@ -497,7 +504,7 @@ def latent_norm_cache(src: torch.Tensor, off: int, R: int, w: torch.Tensor, eps:
 
 
 def latent_attn(qa: torch.Tensor, cache: torch.Tensor, block_tables, cu_q, ctx_lens, window: int,
-                scale: float) -> torch.Tensor:
+                scale: float, max_qlen: int = 0) -> torch.Tensor:
     """Multi-query attention whose keys and values are the cached latent rows (csrc/attention_latent.hip):
     qa fp32 [T, H, R]; sequence b's rows cu_q[b]:cu_q[b+1] sit at positions ctx_lens[b] - qlen .. ctx_lens[b] - 1
     and see the positions j with 0 <= i - j (< window when window > 0). Returns fp32 [T, H, R]."""

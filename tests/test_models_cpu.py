@@ -80,7 +80,7 @@ def test_preemption_keeps_results(ckpts):
 def test_presets_and_params():
     for n in preset_names():
         cfg = get_preset(n)
-        assert cfg.head_dim * cfg.num_heads == cfg.hidden_size or cfg.model_type == "llama"
+        assert cfg.head_dim * cfg.num_heads == cfg.hidden_size or cfg.model_type == "llama" or cfg.layer_specs
     c = get_preset("llama2-7b")
     assert abs(c.num_params() - 6.74e9) / 6.74e9 < 0.01
     c = get_preset("llama2-70b")

@@ -48,6 +48,12 @@ CONFIGS = {
         layer(mixer(4, 4, 4, 8, 0.5, window=20), moe(3, 3, 8, 1.0)),
         layer(mixer(1, 24, 20, 24, 0.2, window=7, kv_from=0), moe(5, 1, 12, 4.0, shared=(8, 0.5))),
     ]),
+    # latent ranks 64 and 128 (in bf16 on a GPU the matrix-core attention kernel runs), windows 33 and 70
+    "wide": dict(architecture="Timisun", vocab=83, width=64, embedding=dict(scale=2.0), norm=dict(eps=1e-6), layers=[
+        layer(mixer(4, 16, 16, 64, 0.25, window=70), moe(4, 2, 32, 3.0, shared=(32, 2.0))),
+        layer(mixer(2, 32, 24, 128, 0.2), None),
+        layer(mixer(5, 16, 8, 64, 0.25, window=33, kv_from=0), moe(8, 2, 16, 2.0)),
+    ]),
     # one head, top 1, window 1 (a token sees itself only), then a window larger than any test sequence
     "ones": dict(architecture="Timisun", vocab=61, width=24, embedding=dict(scale=1.0), norm=dict(eps=1e-6), layers=[
         layer(mixer(1, 8, 8, 8, 1.0, window=1), moe(2, 1, 8, 1.0)),
@@ -163,9 +169,11 @@ def test_prefill_against_token_by_token_decoding(cases, name, device, dtype):
 
 
 @pytest.mark.parametrize("device,dtype", RUNS)
-@pytest.mark.parametrize("cuts", [(2, 2, 2, 3, 5, 16, 17, 2, 1, 1, 9), (15, 1, 16, 1, 17, 6), (33, 2, 21)])
-def test_portions_of_several_sizes(cases, cuts, device, dtype):
-    c = cases("mixed", device, dtype)
+@pytest.mark.parametrize("name", ["mixed", "wide"])
+@pytest.mark.parametrize("cuts", [(2, 2, 2, 3, 5, 16, 17, 2, 1, 1, 9), (15, 1, 16, 1, 17, 6), (33, 2, 21),
+                                  (70, 2, 33, 1, 1, 30)])
+def test_portions_of_several_sizes(cases, cuts, name, device, dtype):
+    c = cases(name, device, dtype)
     t = toks(sum(cuts), c.V, 4)
     eng = c.engine()
     got, at = [], 0
@@ -177,8 +185,9 @@ def test_portions_of_several_sizes(cases, cuts, device, dtype):
 
 
 @pytest.mark.parametrize("device,dtype", RUNS)
-def test_mixed_batch_of_unequal_requests_equals_each_alone(cases, device, dtype):
-    c = cases("mixed", device, dtype)
+@pytest.mark.parametrize("name", ["mixed", "wide"])
+def test_mixed_batch_of_unequal_requests_equals_each_alone(cases, name, device, dtype):
+    c = cases(name, device, dtype)
     seqs = {0: toks(50, c.V, 5), 1: toks(23, c.V, 6), 2: toks(9, c.V, 7), 3: toks(37, c.V, 8)}
     # per step: how many tokens of each request (0 = sits the step out); single tokens ride beside portions
     plan = [{0: 17, 1: 2}, {0: 1, 1: 5, 2: 9}, {0: 1, 1: 16, 3: 30}, {0: 31, 3: 1}, {3: 1, 1: 0}, {3: 5}]
@@ -225,9 +234,10 @@ def test_pages_and_slots_are_used_again(cases, device, dtype):
 
 
 @pytest.mark.parametrize("device,dtype", RUNS)
-def test_long_decoding_past_every_window(cases, device, dtype):
-    c = cases("mixed", device, dtype)
-    t = toks(90, c.V, 30)  # windows 7 and 20 pass over decoded tokens several times; pages of 16 are crossed
+@pytest.mark.parametrize("name", ["mixed", "wide"])
+def test_long_decoding_past_every_window(cases, name, device, dtype):
+    c = cases(name, device, dtype)
+    t = toks(90, c.V, 30)  # every window (7, 20; 33, 70) passes over decoded tokens; pages of 16 are crossed
     eng = c.engine()
     got = [eng.replay_step([(0, t[:5], [4])])]
     got += [eng.replay_step([(0, [tok], [0])]) for tok in t[5:]]
