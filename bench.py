@@ -73,7 +73,21 @@ def main():
                          "reported too), or engine-direct only")
     ap.add_argument("--timeout", type=float, default=float(os.environ.get("LLMSS_BENCH_TIMEOUT_S", "2400")),
                     help="launcher mode: kill every rank and exit 124 after this many seconds")
+    ap.add_argument("--timisun", nargs="?", const="w1024,w2048,w4096", default="",
+                    help="instead of the headline workload: prefill / decode throughput of the Timisun design beside "
+                         "the Llama family at equal size (bench/timisun_compare.py), sizes by name, one GPU")
+    ap.add_argument("--timisun-rounds", type=int, default=2)
     args = ap.parse_args()
+
+    if args.timisun:
+        sys.path.insert(0, os.path.join(ROOT, "bench"))
+        import timisun_compare
+
+        res = timisun_compare.run(args.timisun.split(","), args.batch_per_gpu, args.prompt_len, args.gen_len,
+                                  args.timisun_rounds,
+                                  lambda m: print(f"[bench] {m}", file=sys.stderr, flush=True))
+        print(json.dumps(res), flush=True)
+        return
 
     if args.gpus > 1 and "WORLD_SIZE" not in os.environ:
         sys.exit(launch(args))

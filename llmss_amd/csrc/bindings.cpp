@@ -75,8 +75,10 @@ void launch_dequant_fp8_rows(const void* q, const void* scale, void* w, int64_t 
 // fp32 residual stream, strided / grouped GEMMs in either storage type, latent attention, mixture of experts
 void launch_embed_scaled(const void* ids, const void* table, void* x, int T_, int H, int vocab, float scale, int dt,
                          hipStream_t st);
-void launch_resid_add_norm(void* x, const void* a, int64_t lda, const void* b, int64_t ldb, const void* w, float woff,
-                           float eps, void* y, int64_t ldy, int T_, int H, int dt, hipStream_t st);
+void launch_resid_add_norm(void* x, const void* a, int64_t lda, const void* b, int64_t ldb, const void* ey,
+                           const void* place, const void* wts, int top, const void* shared_, int64_t lds_,
+                           const void* w, float woff, float eps, void* y, int64_t ldy, int T_, int H, int dt,
+                           hipStream_t st);
 void launch_gemm_any(const void* A, const void* B, void* C, int M, int N, int K, int batch, int64_t sAb, int64_t sAm,
                      int64_t sBb, int64_t sBn, int64_t sBk, int64_t sCb, int64_t sCm, int da, int db, int dc,
                      hipStream_t st);
@@ -241,9 +243,11 @@ PYBIND11_MODULE(_C, m) {
   });
   m.def("embed_scaled", [](uintptr_t ids, uintptr_t table, uintptr_t x, int T, int H, int V, float scale, int dt,
                            uintptr_t st) { launch_embed_scaled(CP(ids), CP(table), P(x), T, H, V, scale, dt, S(st)); });
-  m.def("resid_add_norm", [](uintptr_t x, uintptr_t a, int64_t lda, uintptr_t b, int64_t ldb, uintptr_t w, float woff,
-                             float eps, uintptr_t y, int64_t ldy, int T, int H, int dt, uintptr_t st) {
-    launch_resid_add_norm(P(x), CP(a), lda, CP(b), ldb, CP(w), woff, eps, P(y), ldy, T, H, dt, S(st));
+  m.def("resid_add_norm", [](uintptr_t x, uintptr_t a, int64_t lda, uintptr_t b, int64_t ldb, uintptr_t ey,
+                             uintptr_t place, uintptr_t wts, int top, uintptr_t sh, int64_t lds_, uintptr_t w,
+                             float woff, float eps, uintptr_t y, int64_t ldy, int T, int H, int dt, uintptr_t st) {
+    launch_resid_add_norm(P(x), CP(a), lda, CP(b), ldb, CP(ey), CP(place), CP(wts), top, CP(sh), lds_, CP(w), woff,
+                          eps, P(y), ldy, T, H, dt, S(st));
   });
   m.def("gemm_any", [](uintptr_t A, uintptr_t B, uintptr_t C, int M, int N, int K, int batch, int64_t sAb, int64_t sAm,
                        int64_t sBb, int64_t sBn, int64_t sBk, int64_t sCb, int64_t sCm, int da, int db, int dc,

@@ -69,7 +69,9 @@ class MoEFeedForward:
         if W.shared_gu is not None:
             gu = ops.linear_f(h, W.shared_gu, dt)
             sh = ops.linear_f(ops.glu_clamp(gu, spec.shared.ff, spec.shared.limit, GLU_ALPHA), W.shared_down, dt)
-        return ops.moe_experts(h, idx, wts, W.gate, W.up, W.down, spec.expert.limit, GLU_ALPHA, shared=sh)
+        # combine=False: on the GPU the weighted sum over the chosen experts happens inside the next residual add
+        return ops.moe_experts(h, idx, wts, W.gate, W.up, W.down, spec.expert.limit, GLU_ALPHA, shared=sh,
+                               combine=False)
 
 
 MIXERS = {"latent_attention": LatentAttention}

@@ -646,7 +646,8 @@ def load_timisun_weights(cfg: ModelConfig, reader, device="cpu", dtype=torch.bfl
 def random_timisun_weights(cfg: ModelConfig, device="cpu", dtype=torch.bfloat16, seed: int = 0) -> ModelWeights:
     """Random-init weights of a per-layer (Timisun) config: projections ~ N(0, 1 / fan_in), norm weights and the
     router's correction small around zero, values rounded to bf16 (so a bf16 and an fp32 run hold the same model)."""
-    return _timisun_finish(cfg, _timisun_random(cfg, seed), device, dtype)
+    gen = device if torch.device(device).type == "cuda" else "cpu"  # large models: draw on the GPU
+    return _timisun_finish(cfg, _timisun_random(cfg, seed, gen), device, dtype)
 
 
 def timisun_state_dict(cfg: ModelConfig, seed: int = 0) -> Dict[str, torch.Tensor]:
@@ -667,7 +668,7 @@ def timisun_state_dict(cfg: ModelConfig, seed: int = 0) -> Dict[str, torch.Tenso
     return {n: get(n).to(torch.bfloat16) for n in names}
 
 
-def _timisun_random(cfg: ModelConfig, seed: int):
+def _timisun_random(cfg: ModelConfig, seed: int, device="cpu"):
     import zlib
 
     W = cfg.hidden_size
@@ -703,10 +704,10 @@ def _timisun_random(cfg: ModelConfig, seed: int):
         return ((W, e.ff), e.ff ** -0.5) if part == "down" else ((e.ff, W), W ** -0.5)
 
     def get(name: str) -> torch.Tensor:
-        g = torch.Generator()
+        g = torch.Generator(device=device)
         g.manual_seed((seed * 1000003 + zlib.crc32(name.encode())) & 0x7FFFFFFF)
         shp, std = shape_of(name)
-        t = torch.randn(*shp, generator=g, dtype=torch.float32)
+        t = torch.randn(*shp, generator=g, dtype=torch.float32, device=device)
         t = 1.0 + 0.1 * t if std is None else t * std
         return t.to(torch.bfloat16).float()
     return get

@@ -808,6 +808,18 @@ def embed_scaled(ids, table, scale):
     return x
 
 
+class MoEPending:
+    """Expert outputs of a mixture-of-experts layer before they are weighted and summed (``moe_experts(...,
+    combine=False)``): fp32 rows ``y`` [pairs, N] in expert order, ``place`` [T * top] the row of each (token, slot)
+    pair, ``wts`` [T, top], ``shared`` [T, N] or None. resid_add_norm takes it as its fp32 addend and combines while
+    it adds to the stream."""
+
+    __slots__ = ("y", "place", "wts", "shared")
+
+    def __init__(self, y, place, wts, shared):
+        self.y, self.place, self.wts, self.shared = y, place, wts, shared
+
+
 def resid_add_norm(x, a, b, w, woff, eps, out_dtype, want_y=True):
     T, H = x.shape
     _rows(x, "x", dtype=torch.float32)
@@ -815,7 +827,15 @@ def resid_add_norm(x, a, b, w, woff, eps, out_dtype, want_y=True):
     if a is not None:
         _rows(a, "a", H, out_dtype)
         _check(a.shape[0] == T, "a rows")
-    if b is not None:
+    pend = b if isinstance(b, MoEPending) else None
+    if pend is not None:
+        top = pend.wts.shape[1]
+        _check(pend.y.shape == (T * top, H) and pend.y.is_contiguous() and pend.place.numel() == T * top
+               and pend.wts.shape[0] == T, "pending expert outputs do not fit the stream")
+        if pend.shared is not None:
+            _rows(pend.shared, "shared", H, out_dtype)
+        b = None
+    elif b is not None:
         _rows(b, "b", H, torch.float32)
         _check(b.shape[0] == T, "b rows")
     y = None
@@ -823,9 +843,12 @@ def resid_add_norm(x, a, b, w, woff, eps, out_dtype, want_y=True):
         _check(w.dtype == out_dtype and w.is_contiguous() and w.numel() == H, "norm weight")
         y = torch.empty(T, H, dtype=out_dtype, device=x.device)
     _check(out_dtype in _DT, "out dtype bf16 / fp32")
+    sh = pend.shared if pend is not None else None
     lib().resid_add_norm(x.data_ptr(), _ptr(a), a.stride(0) if a is not None else 0, _ptr(b),
-                         b.stride(0) if b is not None else 0, _ptr(w) if want_y else 0, float(woff), float(eps),
-                         _ptr(y), H, T, H, _DT[out_dtype], _stream())
+                         b.stride(0) if b is not None else 0, _ptr(pend.y) if pend else 0,
+                         _ptr(pend.place) if pend else 0, _ptr(pend.wts) if pend else 0,
+                         pend.wts.shape[1] if pend else 0, _ptr(sh), sh.stride(0) if sh is not None else 0,
+                         _ptr(w) if want_y else 0, float(woff), float(eps), _ptr(y), H, T, H, _DT[out_dtype], _stream())
     return y
 
 
@@ -963,7 +986,8 @@ def moe_route(z, corr, top):
     return idx, wts
 
 
-def moe_experts(h, idx, wts, gate, up, down, limit, alpha, shared=None):
+def moe_experts(h, idx, wts, gate, up, down, limit, alpha, shared=None, combine=True):
+    """``combine=False``: leave the weighting and summing to resid_add_norm (returns a :class:`MoEPending`)."""
     T, K = h.shape
     E, F, _ = gate.shape
     N = down.shape[1]
@@ -977,7 +1001,7 @@ def moe_experts(h, idx, wts, gate, up, down, limit, alpha, shared=None):
     if shared is not None:
         _rows(shared, "shared", N, h.dtype)
         _check(shared.shape[0] == T, "shared rows")
-    out = torch.empty(T, N, dtype=torch.float32, device=h.device)
+    out = torch.empty(T, N, dtype=torch.float32, device=h.device) if combine or T == 0 else None
     if T == 0:
         return out
     P = T * top
@@ -1000,6 +1024,8 @@ def moe_experts(h, idx, wts, gate, up, down, limit, alpha, shared=None):
         L.moe_gate_up(h.data_ptr(), h.stride(0), gate.data_ptr(), up.data_ptr(), meta.data_ptr(), order.data_ptr(),
                       act.data_ptr(), E, maxt, top, F, K, float(limit), float(alpha), dt, st)
         L.moe_down(act.data_ptr(), down.data_ptr(), meta.data_ptr(), y.data_ptr(), E, maxt, N, F, dt, st)
+    if not combine:
+        return MoEPending(y, place, wts, shared)
     L.moe_combine(y.data_ptr(), place.data_ptr(), wts.data_ptr(), _ptr(shared),
                   shared.stride(0) if shared is not None else 0, out.data_ptr(), T, N, top, dt, st)
     return out

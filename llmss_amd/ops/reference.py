@@ -556,7 +556,8 @@ def moe_route(z: torch.Tensor, corr: Optional[torch.Tensor], top: int):
 
 
 def moe_experts(h: torch.Tensor, idx: torch.Tensor, wts: torch.Tensor, gate: torch.Tensor, up: torch.Tensor,
-                down: torch.Tensor, limit: float, alpha: float, shared: Optional[torch.Tensor] = None) -> torch.Tensor:
+                down: torch.Tensor, limit: float, alpha: float, shared: Optional[torch.Tensor] = None,
+                combine: bool = True) -> torch.Tensor:
     """sum_j wts[t, j] * down_e(glu(gate_e h, up_e h)) (+ shared) with e = idx[t, j] -> fp32 [T, N]. Stacked expert
     weights gate / up [E, F, K], down [E, N, F]; the activation is rounded to the storage type between the
     products, as the grouped GEMMs do."""
