@@ -270,6 +270,20 @@ __global__ __launch_bounds__(256) void attn_decode_reduce_kernel(const float* __
   }
 }
 
+// The reduce alone, for other kernels that leave partials in the same layout (attention_extend.hip's key split).
+void launch_attn_decode_reduce(const float* part_o, const float* part_ml, void* out, int64_t out_stride, int B, int nh,
+                               int D, int nsplit, hipStream_t st) {
+  if (B == 0) return;
+  dim3 g(B, nh);
+  switch (D) {
+    case 64: attn_decode_reduce_kernel<64><<<g, 64, 0, st>>>(part_o, part_ml, (bf16_t*)out, out_stride, nh, nsplit); break;
+    case 128: attn_decode_reduce_kernel<128><<<g, 128, 0, st>>>(part_o, part_ml, (bf16_t*)out, out_stride, nh, nsplit); break;
+    case 256: attn_decode_reduce_kernel<256><<<g, 256, 0, st>>>(part_o, part_ml, (bf16_t*)out, out_stride, nh, nsplit); break;
+    default: throw std::runtime_error("attn_decode_reduce: head_dim must be 64, 128 or 256");
+  }
+  HIP_CHECK_LAUNCH();
+}
+
 // tokens in flight per (wave, slot): 1 / 2 / 4 = one register set; 11 / 12 / 14 = two register sets,
 // the next set's loads issued before the current set is consumed (tuning knob attn_decode_set_unroll)
 // default 11 (measured, bench/attn_bench.py, cold KV, B = 64: best or within 1% of best for MHA at

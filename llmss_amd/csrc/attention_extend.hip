@@ -20,6 +20,10 @@
 //
 // Sliding window (window > 0): query position p attends keys (p - window, p] only; the key loop starts at the tile
 // holding the first row's oldest visible key, and tiles wholly before a wave's window are skipped.
+// Key split (nsplit > 1, single-token rows only): workgroup x = s handles the s-th run of split_keys keys of its
+// sequence's visible range and leaves the unnormalised O, running maximum and sum in the decode kernel's partial
+// buffers ([token, head, split]); attn_decode_reduce_kernel (attention_decode.hip) joins them. A decode step whose
+// sequences are few but long then fills the chip instead of one workgroup walking each sequence.
 // SAME: keys and values are one tensor (latent attention, where both are the cached latent row and nkv = 1): the
 // tile is loaded and staged once and serves both products.
 #include "common.h"
@@ -37,7 +41,8 @@ __global__ __launch_bounds__(256) void attn_extend_kernel(
     const bf16_t* __restrict__ q, int64_t q_stride, const void* __restrict__ kcv, const void* __restrict__ vcv,
     const int* __restrict__ block_tables, int max_blocks, const int* __restrict__ cu_q, const int* __restrict__ ctx_lens,
     bf16_t* __restrict__ out, int64_t out_stride, int nh, int nkv, int GE, int bs, float scale_log2,
-    unsigned char* __restrict__ q8, float* __restrict__ s8, int window) {
+    unsigned char* __restrict__ q8, float* __restrict__ s8, int window, int nsplit, int split_keys,
+    float* __restrict__ part_o, float* __restrict__ part_ml) {
   static_assert(!(SAME && KV8), "a shared key/value tile is staged from bf16 rows");
   constexpr int BKV = 64;
   constexpr int LD = D + 16;  // padded LDS row (elements): conflict-free b128 rows and tr_b16 columns
@@ -51,7 +56,7 @@ __global__ __launch_bounds__(256) void attn_extend_kernel(
   const int kvh = blockIdx.y / (G / GE);
   const int h0 = kvh * G + (blockIdx.y % (G / GE)) * GE;  // first query head of this workgroup
   const int t0 = cu_q[b], qlen = cu_q[b + 1] - t0;
-  const int r0 = blockIdx.x * rows_per_wg;
+  const int r0 = nsplit > 1 ? 0 : blockIdx.x * rows_per_wg;
   if (r0 >= qlen) return;
   const int ctx = ctx_lens[b];
   const int p0 = ctx - qlen;  // position of the chunk's first token
@@ -79,7 +84,12 @@ __global__ __launch_bounds__(256) void attn_extend_kernel(
   // this wave's slots: rows r0 + (16w)/GE .. r0 + (16w+15)/GE
   const int wave_qhi = p0 + min(qlen - 1, r0 + (16 * w + 15) / GE);
   // first key any row of the workgroup / of this wave may see (tile-aligned start of the key loop)
-  const int kv_begin = window > 0 ? max(0, p0 + r0 - window + 1) / BKV * BKV : 0;
+  int kv_begin = window > 0 ? max(0, p0 + r0 - window + 1) / BKV * BKV : 0;
+  int kv_stop = kv_end;  // end of the key loop (kv_end stays the causal bound of the rows)
+  if (nsplit > 1) {
+    kv_begin += blockIdx.x * split_keys;
+    kv_stop = min(kv_end, kv_begin + split_keys);
+  }
   const int wave_klo = window > 0 ? p0 + min(qlen - 1, r0 + (16 * w) / GE) - window + 1 : 0;
   const int* bt = block_tables + (int64_t)b * max_blocks;
   constexpr int CH = D / 8;
@@ -183,15 +193,15 @@ __global__ __launch_bounds__(256) void attn_extend_kernel(
     }
   };
   if constexpr (PIPE) {
-    if (kv_end > kv_begin) load_tile(kv_begin);
+    if (kv_stop > kv_begin) load_tile(kv_begin);
   }
-  for (int kv0 = kv_begin; kv0 < kv_end; kv0 += BKV) {
+  for (int kv0 = kv_begin; kv0 < kv_stop; kv0 += BKV) {
     __syncthreads();  // every wave is done reading the previous tile
     if constexpr (PIPE) store_tile();
     else stage_direct(kv0);
     __syncthreads();
     if constexpr (PIPE) {
-      if (kv0 + BKV < kv_end) load_tile(kv0 + BKV);
+      if (kv0 + BKV < kv_stop) load_tile(kv0 + BKV);
     }
     if (kv0 > wave_qhi) continue;  // whole tile in this wave's causal future (barriers stay uniform)
     if (kv0 + BKV <= wave_klo) continue;  // whole tile older than this wave's windows
@@ -254,6 +264,18 @@ __global__ __launch_bounds__(256) void attn_extend_kernel(
       }
     }
   }
+  if (nsplit > 1) {  // kernel argument: uniform
+    if (valid) {
+      const int64_t pi = ((int64_t)(t0 + row) * nh + h) * nsplit + blockIdx.x;
+#pragma unroll
+      for (int dt = 0; dt < D / 16; ++dt) *reinterpret_cast<f32x4*>(part_o + pi * D + dt * 16 + 4 * g) = o[dt];
+      if (g == 0) {
+        part_ml[pi * 2] = m;
+        part_ml[pi * 2 + 1] = lsum;
+      }
+    }
+    return;
+  }
   const float inv = lsum > 0.f ? 1.f / lsum : 0.f;
   u16x4 res[D / 16];
   float amax = 0.f;
@@ -292,6 +314,9 @@ __global__ __launch_bounds__(256) void attn_extend_kernel(
   }
 }
 
+void launch_attn_decode_reduce(const float* part_o, const float* part_ml, void* out, int64_t out_stride, int B, int nh,
+                               int D, int nsplit, hipStream_t st);
+
 // GE: largest divisor of the group size G that is <= 64 (slots per workgroup)
 static int extend_group(int G) {
   for (int ge = std::min(G, 64); ge >= 1; --ge)
@@ -302,7 +327,8 @@ static int extend_group(int G) {
 void launch_attn_extend(const void* q, int64_t q_stride, const void* k_cache, const void* v_cache,
                         const void* block_tables, int max_blocks, const void* cu_q, const void* ctx_lens, void* out,
                         int64_t out_stride, int B, int max_qlen, int nh, int nkv, int D, int bs, float scale,
-                        hipStream_t st, bool kv8, void* q8v, void* s8v, int window) {
+                        hipStream_t st, bool kv8, void* q8v, void* s8v, int window, int nsplit, int split_keys,
+                        void* part_o, void* part_ml) {
   if (nh % nkv) throw std::runtime_error("attn_extend: nh must be a multiple of nkv");
   if (B == 0 || max_qlen == 0) return;
   const int G = nh / nkv, GE = extend_group(G);
@@ -313,6 +339,15 @@ void launch_attn_extend(const void* q, int64_t q_stride, const void* k_cache, co
     throw std::runtime_error("attn_extend: the fp8 twin needs one kv head and a power-of-two query group <= 16");
   const int rows = 64 / GE;
   dim3 grid((max_qlen + rows - 1) / rows, nkv * (G / GE), B);
+  if (nsplit > 1) {
+    if (max_qlen != 1 || split_keys <= 0 || split_keys % 64 || !part_o || !part_ml || Q8)
+      throw std::runtime_error("attn_extend: a key split needs single-token rows, whole tiles per split and workspaces");
+    grid.x = nsplit;
+  } else {
+    nsplit = 1;
+  }
+  auto PO = (float*)part_o;
+  auto PML = (float*)part_ml;
   auto Q = (const bf16_t*)q;
   auto K = k_cache;
   auto V = v_cache;
@@ -327,13 +362,13 @@ void launch_attn_extend(const void* q, int64_t q_stride, const void* k_cache, co
   do {                                                                                                           \
     if (kv8)                                                                                                     \
       attn_extend_kernel<D_, true><<<grid, 256, 0, st>>>(Q, q_stride, K, V, BT, max_blocks, CU, CL, O, out_stride, nh, \
-                                                         nkv, GE, bs, sl, Q8, S8, window);                       \
+                                                         nkv, GE, bs, sl, Q8, S8, window, nsplit, split_keys, PO, PML);                       \
     else if (same)                                                                                               \
       attn_extend_kernel<D_, false, true><<<grid, 256, 0, st>>>(Q, q_stride, K, V, BT, max_blocks, CU, CL, O,          \
-                                                                out_stride, nh, nkv, GE, bs, sl, Q8, S8, window); \
+                                                                out_stride, nh, nkv, GE, bs, sl, Q8, S8, window, nsplit, split_keys, PO, PML); \
     else                                                                                                         \
       attn_extend_kernel<D_, false><<<grid, 256, 0, st>>>(Q, q_stride, K, V, BT, max_blocks, CU, CL, O, out_stride,   \
-                                                          nh, nkv, GE, bs, sl, Q8, S8, window);                  \
+                                                          nh, nkv, GE, bs, sl, Q8, S8, window, nsplit, split_keys, PO, PML);                  \
   } while (0)
   switch (D) {
     case 64: LX(64); break;
@@ -343,4 +378,8 @@ void launch_attn_extend(const void* q, int64_t q_stride, const void* k_cache, co
   }
 #undef LX
   HIP_CHECK_LAUNCH();
+  if (nsplit > 1) {
+    // B single-token rows: token index = sequence index only when cu_q is 0, 1, .., B (the caller's contract)
+    launch_attn_decode_reduce(PO, PML, out, out_stride, B, nh, D, nsplit, st);
+  }
 }

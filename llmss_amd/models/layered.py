@@ -53,7 +53,8 @@ class LatentAttention:
             ops.latent_norm_cache(qc, H * dim, R, W.kv_norm, model.cfg.norm_eps, cache, inp.slots)
         qa = ops.head_absorb(qc, W.uk_t, ops.latent_qa_dtype(cache))
         o = ops.latent_attn(qa, cache, inp.block_tables, cu, inp.ctx_lens, spec.window, spec.scale,
-                            max_qlen=1 if inp.kind == "decode" else max(1, inp.max_seqlen))
+                            max_qlen=1 if inp.kind == "decode" else max(1, inp.max_seqlen),
+                            max_ctx=inp.max_ctx if inp.kind == "decode" else 0)
         return ops.linear_f(ops.head_expand(o, W.uv, dt), W.o, dt)
 
 

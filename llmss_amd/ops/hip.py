@@ -194,8 +194,10 @@ def extend_fp8_twin_ok(nh: int, nkv: int) -> bool:
 
 
 def attn_extend(q, k_cache, v_cache, block_tables, cu_q, ctx_lens, max_qlen, nh, nkv, D, scale, out=None,
-                fp8_out=False, window=0):
-    """Chunked-prefill attention: q rows [T, >= nh*D] (query heads first, as in the QKV output) of B
+                fp8_out=False, window=0, key_split=None):
+    """``key_split`` = (nsplit, keys per split, a multiple of 64): single-token rows only (cu_q = 0, 1, .., B) - the
+    visible keys of each row are cut over nsplit workgroups whose partials a reduce kernel joins.
+    Chunked-prefill attention: q rows [T, >= nh*D] (query heads first, as in the QKV output) of B
     sequences (``cu_q`` [B+1] int32), each attending its whole paged context ``ctx_lens`` [B] int32 (the
     chunk's own K/V already written to the cache) causally; ``window`` > 0 limits a position to itself and the
     ``window - 1`` positions before it. ``fp8_out`` (only where extend_fp8_twin_ok):
@@ -220,9 +222,15 @@ def attn_extend(q, k_cache, v_cache, block_tables, cu_q, ctx_lens, max_qlen, nh,
     if fp8_out:
         _check(extend_fp8_twin_ok(nh, nkv) and y.shape == (T, nh * D), "fp8 twin: one kv head, group <= 16, dense out")
         q8, s8 = _fp8_twin(y)
+    nsplit, split_keys, po, pml = 1, 0, None, None
+    if key_split is not None and key_split[0] > 1:
+        nsplit, split_keys = int(key_split[0]), int(key_split[1])
+        _check(max_qlen == 1 and T == B and split_keys % 64 == 0 and not fp8_out, "key split: single-token rows")
+        po, pml = _DECODE_WS.get(T, nh, nsplit, D, q.device)
     lib().attn_extend(q.data_ptr(), q.stride(0), k_cache.data_ptr(), v_cache.data_ptr(), block_tables.data_ptr(),
                       block_tables.shape[1], cu_q.data_ptr(), ctx_lens.data_ptr(), y.data_ptr(), y.stride(0), B,
-                      int(max_qlen), nh, nkv, D, bs, float(scale), _stream(), kv8, _ptr(q8), _ptr(s8), int(window))
+                      int(max_qlen), nh, nkv, D, bs, float(scale), _stream(), kv8, _ptr(q8), _ptr(s8), int(window),
+                      nsplit, split_keys, _ptr(po), _ptr(pml))
     return y
 
 
@@ -936,7 +944,17 @@ def latent_qa_dtype(cache) -> torch.dtype:
     return torch.float32
 
 
-def latent_attn(qa, cache, block_tables, cu_q, ctx_lens, window, scale, max_qlen=0):
+def latent_key_split(B: int, window: int, max_ctx: int):
+    """(nsplit, keys per split) for a decode step of B single-token rows whose visible range is at most
+    min(window, max_ctx) keys: about 1024 workgroups in flight, whole 64-key tiles per split."""
+    keys = min(window, max_ctx) if window > 0 else max_ctx
+    tiles = -(-keys // 64) + (1 if window > 0 else 0)  # a window may straddle one more tile
+    nsplit = max(1, min(tiles, 1024 // max(1, B)))
+    per = -(-tiles // nsplit)
+    return -(-tiles // per), per * 64
+
+
+def latent_attn(qa, cache, block_tables, cu_q, ctx_lens, window, scale, max_qlen=0, max_ctx=0):
     """``qa`` [T, H, R]. bf16 queries over a bf16 cache of rank 64 / 128 / 256 run the MFMA extend kernel as
     multi-query attention whose one key/value head is the latent row (keys = values = cache, bf16 output); anything
     else runs the generic kernel (fp32 queries, fp32 output)."""
@@ -950,8 +968,9 @@ def latent_attn(qa, cache, block_tables, cu_q, ctx_lens, window, scale, max_qlen
     if qa.dtype == torch.bfloat16:
         _check(latent_qa_dtype(cache) == torch.bfloat16 and max_qlen > 0, "bf16 queries: MFMA ranks and max_qlen only")
         kv = cache.view(cache.shape[0], 1, cache.shape[1], R)  # [blocks, one kv head, block_size, R]
+        split = latent_key_split(T, window, max_ctx) if max_qlen == 1 and T == B and max_ctx > 0 else None
         out = attn_extend(qa.view(T, H * R), kv, kv, block_tables, cu_q, ctx_lens[:B], max_qlen, H, 1, R, scale,
-                          window=window)
+                          window=window, key_split=split)
         return out.view(T, H, R)
     _check(qa.dtype == torch.float32, "qa fp32")
     _check(R <= 512, "latent rank above 512")

@@ -504,7 +504,7 @@ def latent_norm_cache(src: torch.Tensor, off: int, R: int, w: torch.Tensor, eps:
 
 
 def latent_attn(qa: torch.Tensor, cache: torch.Tensor, block_tables, cu_q, ctx_lens, window: int,
-                scale: float, max_qlen: int = 0) -> torch.Tensor:
+                scale: float, max_qlen: int = 0, max_ctx: int = 0) -> torch.Tensor:
     """Multi-query attention whose keys and values are the cached latent rows (csrc/attention_latent.hip):
     qa fp32 [T, H, R]; sequence b's rows cu_q[b]:cu_q[b+1] sit at positions ctx_lens[b] - qlen .. ctx_lens[b] - 1
     and see the positions j with 0 <= i - j (< window when window > 0). Returns fp32 [T, H, R]."""

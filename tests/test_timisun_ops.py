@@ -64,7 +64,8 @@ def run_attention(device, dtype, h, c, wq, wuk, wuv, wo, heads, dim, vdim, scale
         uk_t = d(wuk.view(heads, dim, R).transpose(1, 2).contiguous())
         qa = ops.head_absorb(q, uk_t, ops.latent_qa_dtype(cache))
         o = ops.latent_attn(qa, cache, bt, torch.tensor([0, n], dtype=torch.int32, device=device),
-                            torch.tensor([at + n], dtype=torch.int32, device=device), window, scale, max_qlen=n)
+                            torch.tensor([at + n], dtype=torch.int32, device=device), window, scale, max_qlen=n,
+                            max_ctx=T + 70 if n == 1 else 0)  # a decoded row: its keys may be split over workgroups
         out.append(ops.linear_f(ops.head_expand(o, d(wuv), dtype), d(wo), dtype))
         at += n
     return torch.cat(out)
