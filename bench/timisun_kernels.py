@@ -58,13 +58,15 @@ def main():
     rows = []
 
     def add(name, phase, sec, flops=0.0, bytes_=0.0, like=None):
+        """``of_roofline``: the time the kernel's own roofline allows - the larger of flops / peak matrix rate and
+        bytes / peak HBM rate - over the time measured."""
         r = dict(kernel=name, phase=phase, us=round(sec * 1e6, 1))
         if flops:
             r["tflops"] = round(flops / sec / 1e12, 1)
-            r["of_peak"] = round(flops / sec / 1e12 / PEAK_TFLOPS, 4)
         if bytes_:
             r["tb_s"] = round(bytes_ / sec / 1e12, 3)
-            r["of_peak"] = round(bytes_ / sec / 1e12 / PEAK_TBS, 4)
+        if flops or bytes_:
+            r["of_roofline"] = round(max(flops / (PEAK_TFLOPS * 1e12), bytes_ / (PEAK_TBS * 1e12)) / sec, 4)
         if like:
             r["like"] = like
         rows.append(r)
@@ -82,13 +84,16 @@ def main():
         # ---------------- per-head absorbed / expanded projections vs a dense GEMM of similar work
         q, uk_t = rn(M, Hh * dim, std=0.3), rn(Hh, R, dim, std=dim ** -0.5)
         t = timed(lambda: ops.head_absorb(q, uk_t, bf))
-        add("head_absorb (gemm_tile, batched)", phase, t, flops=2.0 * M * Hh * dim * R)
+        add("head_absorb (gemm_tile, batched)", phase, t, flops=2.0 * M * Hh * dim * R,
+            bytes_=2.0 * (M * Hh * dim + M * Hh * R + Hh * R * dim))
         o, uv = rn(M, Hh, R, std=0.3), rn(Hh * vd, R, std=R ** -0.5)
         t = timed(lambda: ops.head_expand(o, uv, bf))
-        add("head_expand (gemm_tile, batched)", phase, t, flops=2.0 * M * Hh * R * vd)
+        add("head_expand (gemm_tile, batched)", phase, t, flops=2.0 * M * Hh * R * vd,
+            bytes_=2.0 * (M * Hh * R + M * Hh * vd + Hh * vd * R))
         h, wo = rn(M, W, std=0.3), rn(W, W, std=W ** -0.5)
         t = timed(lambda: ops.linear(h, wo))
-        add("dense o-projection (gemm.hip)", phase, t, flops=2.0 * M * W * W, like="head_absorb / head_expand")
+        add("dense o-projection (gemm.hip)", phase, t, flops=2.0 * M * W * W, bytes_=2.0 * (2 * M * W + W * W),
+            like="head_absorb / head_expand")
         # ---------------- experts vs dense gated MLP
         router, corr = rn(E, W, std=W ** -0.5), rn(E, dt=torch.float32, std=0.1)
         gate, up, down = rn(E, F, W, std=W ** -0.5), rn(E, F, W, std=W ** -0.5), rn(E, W, F, std=F ** -0.5)
@@ -99,12 +104,12 @@ def main():
         t = timed(lambda: ops.moe_experts(h, idx, wts, gate, up, down, 7.0, 1.702, combine=False))
         touched = min(E, M * top)
         add("experts: group + gate_up + down (gemm_tile grouped)", phase, t, flops=6.0 * M * top * F * W,
-            **({"bytes_": touched * 3 * F * W * 2} if phase == "decode" else {}))
+            bytes_=touched * 3 * F * W * 2 + M * top * (F * 2 * 2 + W * 4) + M * W * 2)
         wu = ops.glu_interleave(rn(Fd, W, std=W ** -0.5), rn(Fd, W, std=W ** -0.5), 0)
         wd = rn(W, Fd, std=Fd ** -0.5)
         t = timed(lambda: ops.linear(ops.linear(h, wu, None, "none", True), wd))
         add("dense gated MLP (gemm.hip, 2 launches)", phase, t, flops=6.0 * M * Fd * W,
-            **({"bytes_": 3 * Fd * W * 2} if phase == "decode" else {}), like="experts")
+            bytes_=3 * Fd * W * 2 + M * (Fd * 2 * 2 + W * 2 * 2), like="experts")
     # ---------------- attention, prompt: B sequences of `seq` tokens
     bs = 16
     B, S = max(1, a.tokens // a.seq), a.seq
@@ -116,17 +121,18 @@ def main():
     qa = rn(B * S, Hh, R, std=0.1)
     t = timed(lambda: ops.latent_attn(qa, cache, bt, cu, ctx, win, dim ** -0.5, max_qlen=S))
     pairs = sum(min(i + 1, win) for i in range(S)) * B
-    add(f"latent attention, prompt (extend kernel, rank {R}, window {win})", "prompt", t, flops=4.0 * Hh * R * pairs)
+    add(f"latent attention, prompt (extend kernel, rank {R}, window {win})", "prompt", t, flops=4.0 * Hh * R * pairs,
+        bytes_=2.0 * (2 * B * S * Hh * R + B * S * R))
     D = W // Hh
     qkv = rn(B * S, 3 * Hh * D, std=0.3)
     t = timed(lambda: ops.attn_prefill(qkv, cu, S, Hh, Hh, D, D ** -0.5))
     add(f"dense causal attention, prompt (head_dim {D})", "prompt", t, flops=4.0 * Hh * D * B * S * (S + 1) / 2,
-        like="latent attention, prompt")
+        bytes_=2.0 * 4 * B * S * Hh * D, like="latent attention, prompt")
     # ---------------- attention, decode: `batch` sequences with `ctx` cached tokens
     B, C = a.batch, a.ctx
     nblk = -(-C // bs)
     cache = rn(B * nblk, bs, R, std=0.3)
-    bt = torch.arange(B * nblk, dtype=torch.int32, device=dev).view(B, nblk)
+    bt = torch.nn.functional.pad(torch.arange(B * nblk, dtype=torch.int32, device=dev).view(B, nblk), (0, 8))
     cu = torch.arange(B + 1, dtype=torch.int32, device=dev)
     ctx = torch.full((B,), C, dtype=torch.int32, device=dev)
     qa = rn(B, Hh, R, std=0.1)

@@ -87,16 +87,17 @@ void launch_gemm_tile(const void* A, const void* B, void* C, int M, int N, int K
                       int64_t sBb, int64_t sBn, int64_t sCb, int64_t sCm, int dc, hipStream_t st);
 void launch_moe_gate_up_tile(const void* h, int64_t ldh, const void* wg, const void* wu, const void* meta,
                              const void* order, void* act, int E, int maxt, int top, int F, int K, float limit,
-                             float alpha, hipStream_t st);
+                             float alpha, int tile_rows, hipStream_t st);
 void launch_moe_down_tile(const void* act, const void* wd, const void* meta, void* y, int E, int maxt, int N, int F,
-                          hipStream_t st);
+                          int tile_rows, hipStream_t st);
 void launch_latent_norm_cache(const void* src, int64_t ld, int off, const void* w, float eps, void* cache,
                               const void* slots, int T_, int R, int dt, hipStream_t st);
 void launch_latent_attn(const void* qa, int64_t ldq, const void* cache, const void* bt, int maxb, const void* cu_q,
                         const void* ctx_lens, void* out, int64_t ldo, int T_, int B, int H, int R, int bs, int window,
                         float scale, int dt, hipStream_t st);
 void launch_moe_route(const void* z, const void* corr, void* idx, void* wts, int T_, int E, int top, hipStream_t st);
-void launch_moe_group(const void* idx, int P, int E, int maxt, void* meta, void* order, void* place, hipStream_t st);
+void launch_moe_group(const void* idx, int P, int E, int maxt, void* meta, void* order, void* place, int tile_rows,
+                      hipStream_t st);
 void launch_moe_gate_up(const void* h, int64_t ldh, const void* wg, const void* wu, const void* meta,
                         const void* order, void* act, int E, int maxt, int top, int F, int K, float limit,
                         float alpha, int dt, hipStream_t st);
@@ -263,12 +264,14 @@ PYBIND11_MODULE(_C, m) {
   });
   m.def("moe_gate_up_tile", [](uintptr_t h, int64_t ldh, uintptr_t wg, uintptr_t wu, uintptr_t meta, uintptr_t order,
                                uintptr_t act, int E, int maxt, int top, int F, int K, float limit, float alpha,
-                               uintptr_t st) {
+                               int tile_rows, uintptr_t st) {
     launch_moe_gate_up_tile(CP(h), ldh, CP(wg), CP(wu), CP(meta), CP(order), P(act), E, maxt, top, F, K, limit, alpha,
-                            S(st));
+                            tile_rows, S(st));
   });
   m.def("moe_down_tile", [](uintptr_t act, uintptr_t wd, uintptr_t meta, uintptr_t y, int E, int maxt, int N, int F,
-                            uintptr_t st) { launch_moe_down_tile(CP(act), CP(wd), CP(meta), P(y), E, maxt, N, F, S(st)); });
+                            int tile_rows, uintptr_t st) {
+    launch_moe_down_tile(CP(act), CP(wd), CP(meta), P(y), E, maxt, N, F, tile_rows, S(st));
+  });
   m.def("latent_norm_cache", [](uintptr_t src, int64_t ld, int off, uintptr_t w, float eps, uintptr_t cache,
                                 uintptr_t slots, int T, int R, int dt, uintptr_t st) {
     launch_latent_norm_cache(CP(src), ld, off, CP(w), eps, P(cache), CP(slots), T, R, dt, S(st));
@@ -282,7 +285,9 @@ PYBIND11_MODULE(_C, m) {
   m.def("moe_route", [](uintptr_t z, uintptr_t corr, uintptr_t idx, uintptr_t wts, int T, int E, int top,
                         uintptr_t st) { launch_moe_route(CP(z), CP(corr), P(idx), P(wts), T, E, top, S(st)); });
   m.def("moe_group", [](uintptr_t idx, int Pn, int E, int maxt, uintptr_t meta, uintptr_t order, uintptr_t place,
-                        uintptr_t st) { launch_moe_group(CP(idx), Pn, E, maxt, P(meta), P(order), P(place), S(st)); });
+                        int tile_rows, uintptr_t st) {
+    launch_moe_group(CP(idx), Pn, E, maxt, P(meta), P(order), P(place), tile_rows, S(st));
+  });
   m.def("moe_gate_up", [](uintptr_t h, int64_t ldh, uintptr_t wg, uintptr_t wu, uintptr_t meta, uintptr_t order,
                           uintptr_t act, int E, int maxt, int top, int F, int K, float limit, float alpha, int dt,
                           uintptr_t st) {

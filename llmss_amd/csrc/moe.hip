@@ -4,8 +4,8 @@
 //   moe_route:   s = sigmoid(z); the `top` experts with the largest s + correction are chosen (ties: the lower
 //                index); weights = chosen s / (their sum + 1e-20)     -> idx [T, top] int32, wts [T, top] fp32
 //   moe_group:   pairs p = t * top + j are bucketed by expert: off [E + 1], order [P] (pair at each sorted row),
-//                place [P] (sorted row of each pair) and a flat list of 64-row tiles (expert, first row) so the
-//                grouped GEMMs launch a grid whose size is known on the host (ceil(P / 64) + E tiles at most)
+//                place [P] (sorted row of each pair) and a flat list of row tiles (expert, first row; 64 or 128 rows each) so the
+//                grouped GEMMs launch a grid whose size is known on the host (ceil(P / rows) + E tiles at most)
 //   moe_gate_up: act[r, f] = glu(h[token(r)] . gate_e[f], h[token(r)] . up_e[f])   for sorted row r of expert e
 //   moe_down:    y[r, n] = act[r, :] . down_e[n, :]                   (fp32)
 //   moe_combine: out[t, :] = sum_j wts[t, j] * y[place[t * top + j], :] (+ shared[t, :])   (fp32, j ascending)
@@ -85,7 +85,7 @@ void launch_moe_route(const void* z, const void* corr, void* idx, void* wts, int
 // One workgroup. meta = [ntiles | off[E + 1] | tile_expert[maxt] | tile_row0[maxt]], order [P], place [P].
 __global__ __launch_bounds__(1024) void moe_group_kernel(const int* __restrict__ idx, int P, int E, int maxt,
                                                          int* __restrict__ meta, int* __restrict__ order,
-                                                         int* __restrict__ place) {
+                                                         int* __restrict__ place, int tile_rows) {
   extern __shared__ int sm[];  // cnt[E], cur[E]
   int* cnt = sm;
   int* cur = sm + E;
@@ -101,7 +101,7 @@ __global__ __launch_bounds__(1024) void moe_group_kernel(const int* __restrict__
     for (int e = 0; e < E; ++e) {
       off[e] = o;
       cur[e] = o;
-      for (int r = 0; r < cnt[e]; r += TV_BM) {
+      for (int r = 0; r < cnt[e]; r += tile_rows) {
         if (nt < maxt) {
           tile_e[nt] = e;
           tile_r[nt] = o + r;
@@ -123,11 +123,13 @@ __global__ __launch_bounds__(1024) void moe_group_kernel(const int* __restrict__
   }
 }
 
-void launch_moe_group(const void* idx, int P, int E, int maxt, void* meta, void* order, void* place, hipStream_t st) {
+void launch_moe_group(const void* idx, int P, int E, int maxt, void* meta, void* order, void* place, int tile_rows,
+                      hipStream_t st) {
   if (P == 0) return;
+  if (tile_rows <= 0) throw std::runtime_error("moe_group: tile rows");
   if (E > 4096) throw std::runtime_error("moe_group: more than 4096 experts");
   moe_group_kernel<<<1, 1024, 2 * E * sizeof(int), st>>>((const int*)idx, P, E, maxt, (int*)meta, (int*)order,
-                                                          (int*)place);
+                                                          (int*)place, tile_rows);
   HIP_CHECK_LAUNCH();
 }
 

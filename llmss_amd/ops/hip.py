@@ -1024,7 +1024,9 @@ def moe_experts(h, idx, wts, gate, up, down, limit, alpha, shared=None, combine=
     if T == 0:
         return out
     P = T * top
-    maxt = -(-P // 64) + min(E, P)
+    # rows per tile of the grouped GEMMs: 128 where the experts get enough rows to fill big tiles (bf16 only)
+    rows = 128 if h.dtype == torch.bfloat16 and P >= 128 * E else 64
+    maxt = -(-P // rows) + min(E, P)
     _check(maxt <= 65535, "too many (token, expert) pairs in one step")
     dev = h.device
     meta = torch.empty(1 + (E + 1) + 2 * maxt, dtype=torch.int32, device=dev)
@@ -1034,11 +1036,11 @@ def moe_experts(h, idx, wts, gate, up, down, limit, alpha, shared=None, combine=
     y = torch.empty(P, N, dtype=torch.float32, device=dev)
     L = lib()
     st = _stream()
-    L.moe_group(idx.data_ptr(), P, E, maxt, meta.data_ptr(), order.data_ptr(), place.data_ptr(), st)
+    L.moe_group(idx.data_ptr(), P, E, maxt, meta.data_ptr(), order.data_ptr(), place.data_ptr(), rows, st)
     if h.dtype == torch.bfloat16:  # matrix cores (csrc/gemm_tile.hip)
         L.moe_gate_up_tile(h.data_ptr(), h.stride(0), gate.data_ptr(), up.data_ptr(), meta.data_ptr(),
-                           order.data_ptr(), act.data_ptr(), E, maxt, top, F, K, float(limit), float(alpha), st)
-        L.moe_down_tile(act.data_ptr(), down.data_ptr(), meta.data_ptr(), y.data_ptr(), E, maxt, N, F, st)
+                           order.data_ptr(), act.data_ptr(), E, maxt, top, F, K, float(limit), float(alpha), rows, st)
+        L.moe_down_tile(act.data_ptr(), down.data_ptr(), meta.data_ptr(), y.data_ptr(), E, maxt, N, F, rows, st)
     else:
         L.moe_gate_up(h.data_ptr(), h.stride(0), gate.data_ptr(), up.data_ptr(), meta.data_ptr(), order.data_ptr(),
                       act.data_ptr(), E, maxt, top, F, K, float(limit), float(alpha), dt, st)
