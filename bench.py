@@ -77,6 +77,7 @@ def main():
                     help="instead of the headline workload: prefill / decode throughput of the Timisun design beside "
                          "the Llama family at equal size (bench/timisun_compare.py), sizes by name, one GPU")
     ap.add_argument("--timisun-rounds", type=int, default=2)
+    ap.add_argument("--timisun-kinds", default="timisun,dense", help="which of the two models --timisun runs")
     args = ap.parse_args()
 
     if args.timisun:
@@ -85,7 +86,8 @@ def main():
 
         res = timisun_compare.run(args.timisun.split(","), args.batch_per_gpu, args.prompt_len, args.gen_len,
                                   args.timisun_rounds,
-                                  lambda m: print(f"[bench] {m}", file=sys.stderr, flush=True))
+                                  lambda m: print(f"[bench] {m}", file=sys.stderr, flush=True),
+                                  kinds=tuple(args.timisun_kinds.split(",")))
         print(json.dumps(res), flush=True)
         return
 

@@ -85,21 +85,22 @@ def measure(model, batch, prompt_len, gen_len, rounds, progress):
     return {k: round(v, 2) for k, v in out.items()}
 
 
-def run(sizes, batch, prompt_len, gen_len, rounds, progress):
+def run(sizes, batch, prompt_len, gen_len, rounds, progress, kinds=("timisun", "dense")):
     dev = torch.device("cuda", torch.cuda.current_device())
     rows = []
     for name in sizes:
         s = SIZES[name]
         row = dict(size=name, shape=s, batch=batch, prompt_len=prompt_len, gen_len=gen_len)
-        for kind in ("timisun", "dense"):
+        for kind in kinds:
             progress(f"{name} {kind}: building")
             model = build(kind, s, dev)
             row[kind] = measure(model, batch, prompt_len, gen_len, rounds, progress)
             row[kind]["params_M"] = round(model.cfg.num_params() / 1e6, 1)
             del model
             torch.cuda.empty_cache()
-        row["prefill_ratio"] = round(row["timisun"]["prefill_tok_s"] / row["dense"]["prefill_tok_s"], 3)
-        row["decode_ratio"] = round(row["timisun"]["decode_tok_s"] / row["dense"]["decode_tok_s"], 3)
+        if "timisun" in row and "dense" in row:
+            row["prefill_ratio"] = round(row["timisun"]["prefill_tok_s"] / row["dense"]["prefill_tok_s"], 3)
+            row["decode_ratio"] = round(row["timisun"]["decode_tok_s"] / row["dense"]["decode_tok_s"], 3)
         rows.append(row)
     return dict(metric="timisun_vs_dense_tokens_per_sec", unit="tokens/s", dtype="bf16", data="synthetic",
                 sizes=rows)

@@ -96,6 +96,8 @@ void launch_latent_attn(const void* qa, int64_t ldq, const void* cache, const vo
                         const void* ctx_lens, void* out, int64_t ldo, int T_, int B, int H, int R, int bs, int window,
                         float scale, int dt, hipStream_t st);
 void launch_moe_route(const void* z, const void* corr, void* idx, void* wts, int T_, int E, int top, hipStream_t st);
+void launch_moe_router(const void* h, int64_t ldh, const void* wr, const void* corr, void* idx, void* wts, int T_,
+                       int E, int K, int top, int dt, hipStream_t st);
 void launch_moe_group(const void* idx, int P, int E, int maxt, void* meta, void* order, void* place, int tile_rows,
                       hipStream_t st);
 void launch_moe_gate_up(const void* h, int64_t ldh, const void* wg, const void* wu, const void* meta,
@@ -284,6 +286,10 @@ PYBIND11_MODULE(_C, m) {
   });
   m.def("moe_route", [](uintptr_t z, uintptr_t corr, uintptr_t idx, uintptr_t wts, int T, int E, int top,
                         uintptr_t st) { launch_moe_route(CP(z), CP(corr), P(idx), P(wts), T, E, top, S(st)); });
+  m.def("moe_router", [](uintptr_t h, int64_t ldh, uintptr_t wr, uintptr_t corr, uintptr_t idx, uintptr_t wts, int T,
+                         int E, int K, int top, int dt, uintptr_t st) {
+    launch_moe_router(CP(h), ldh, CP(wr), CP(corr), P(idx), P(wts), T, E, K, top, dt, S(st));
+  });
   m.def("moe_group", [](uintptr_t idx, int Pn, int E, int maxt, uintptr_t meta, uintptr_t order, uintptr_t place,
                         int tile_rows, uintptr_t st) {
     launch_moe_group(CP(idx), Pn, E, maxt, P(meta), P(order), P(place), tile_rows, S(st));

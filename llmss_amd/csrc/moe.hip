@@ -81,6 +81,82 @@ void launch_moe_route(const void* z, const void* corr, void* idx, void* wts, int
   HIP_CHECK_LAUNCH();
 }
 
+// Router logits and routing in one launch, for steps of few tokens (a decode step): one workgroup per token, its four
+// waves share the experts' dot products z_e = h . W_r[e] (fp32 accumulation over lanes), then the token is routed
+// as moe_route_kernel does. A prompt's thousands of tokens take the matrix-core GEMM and moe_route instead.
+template <typename T>
+__global__ __launch_bounds__(256) void moe_router_kernel(const T* __restrict__ h, int64_t ldh, const T* __restrict__ wr,
+                                                         const float* __restrict__ corr, int* __restrict__ idx,
+                                                         float* __restrict__ wts, int E, int K, int top, bool vec) {
+  extern __shared__ float sc[];  // [E] scores, [E] choice values
+  float* ch = sc + E;
+  const int t = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+  const T* x = h + (int64_t)t * ldh;
+  for (int e = wv; e < E; e += 4) {
+    const T* w = wr + (int64_t)e * K;
+    float acc = 0.f;
+    if (vec) {  // K % 8 == 0, rows 16-byte aligned (bf16) - eight elements per lane and access
+      for (int k = lane * 8; k < K; k += 512) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) acc = fmaf(El<T>::ld(x + k + i), El<T>::ld(w + k + i), acc);
+      }
+    } else {
+      for (int k = lane; k < K; k += 64) acc = fmaf(El<T>::ld(x + k), El<T>::ld(w + k), acc);
+    }
+    acc = warp_sum(acc);
+    if (lane == 0) {
+      const float s = 1.f / (1.f + expf(-acc));
+      sc[e] = s;
+      ch[e] = s + (corr ? corr[e] : 0.f);
+    }
+  }
+  __syncthreads();
+  float sum = 0.f;
+  for (int j = 0; j < top; ++j) {
+    float best = -INFINITY;
+    int bi = 0x7fffffff;
+    for (int e = lane; e < E; e += 64) {
+      const float v = ch[e];
+      if (v > best || (v == best && e < bi)) {
+        best = v;
+        bi = e;
+      }
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+      const float ov = __shfl_xor(best, o, 64);
+      const int oi = __shfl_xor(bi, o, 64);
+      if (ov > best || (ov == best && oi < bi)) {
+        best = ov;
+        bi = oi;
+      }
+    }
+    if (bi >= E) bi = 0;
+    const float s = sc[bi];
+    sum += s;
+    __syncthreads();  // every wave has read ch before the winner is struck out
+    if (tid == 0) {
+      idx[(int64_t)t * top + j] = bi;
+      wts[(int64_t)t * top + j] = s;
+      ch[bi] = -INFINITY;
+    }
+    __syncthreads();
+  }
+  const float inv = 1.f / (sum + 1e-20f);
+  for (int j = tid; j < top; j += 256) wts[(int64_t)t * top + j] *= inv;
+}
+
+void launch_moe_router(const void* h, int64_t ldh, const void* wr, const void* corr, void* idx, void* wts, int T_,
+                       int E, int K, int top, int dt, hipStream_t st) {
+  if (T_ == 0) return;
+  if (top > E || top <= 0) throw std::runtime_error("moe_router: top must be in [1, experts]");
+  const int es = dt == 0 ? 2 : 4;
+  const bool vec = K % 8 == 0 && ((uintptr_t)h % 16) == 0 && ((uintptr_t)wr % 16) == 0 && (ldh * es) % 16 == 0;
+  DISPATCH_T(dt, T, (moe_router_kernel<T><<<T_, 256, 2 * E * sizeof(float), st>>>(
+                        (const T*)h, ldh, (const T*)wr, (const float*)corr, (int*)idx, (float*)wts, E, K, top, vec)));
+  HIP_CHECK_LAUNCH();
+}
+
 // ------------------------------------------------------------------------------------------------ grouping
 // One workgroup. meta = [ntiles | off[E + 1] | tile_expert[maxt] | tile_row0[maxt]], order [P], place [P].
 __global__ __launch_bounds__(1024) void moe_group_kernel(const int* __restrict__ idx, int P, int E, int maxt,

@@ -16,7 +16,7 @@ and attends with the key projection absorbed into the query: qa_h = W_uk_h^T q_h
 over the causal (optionally windowed) keys, out = W_o concat_h(W_uv_h sum_j p_j c_j). A layer with ``kv_from``
 projects no latent of its own and reads the named layer's cache with its own W_uk / W_uv.
 
-Feed-forward ``moe`` (ops: linear_f -> fp32 router logits, moe_route, moe_experts, glu_clamp): sigmoid scores, the
+Feed-forward ``moe`` (ops: moe_router -> fp32 router logits and routing, moe_experts, glu_clamp): sigmoid scores, the
 choice made on score + correction, weights = chosen scores normalised; experts and the shared expert use the clamped
 gated activation g * sigmoid(1.702 g) * (u + 1).
 """
@@ -64,8 +64,7 @@ class MoEFeedForward:
     @staticmethod
     def forward(model: "LayeredLM", W, spec, h):
         dt = model.dtype
-        z = ops.linear_f(h, W.router, torch.float32)
-        idx, wts = ops.moe_route(z, W.correction, spec.top)
+        idx, wts = ops.moe_router(h, W.router, W.correction, spec.top)
         sh = None
         if W.shared_gu is not None:
             gu = ops.linear_f(h, W.shared_gu, dt)

@@ -19,8 +19,9 @@ import torch
 
 from ..parallel.dist import TPGroup
 from .config import ModelConfig
-from .decoder import DecoderLM, StepInput
-from .weights import load_hf_weights
+from .decoder import StepInput
+from .layered import create_model
+from .weights import load_hf_weights, load_timisun_weights
 
 
 @dataclass
@@ -52,8 +53,11 @@ class CausalLM:
     def __init__(self, config, weights, max_blocks: int = 4096, block_size: int = 16):
         cfg = config if isinstance(config, ModelConfig) else ModelConfig.from_hf_dict(config.to_dict())
         tp = getattr(weights, "tp", None) or TPGroup()
-        w = load_hf_weights(cfg, weights.reader, tp.size, tp.rank, device=weights.device, dtype=weights.dtype)
-        self.model = DecoderLM(cfg, w, tp)
+        if cfg.layer_specs:  # per-layer designs (Timisun)
+            w = load_timisun_weights(cfg, weights.reader, device=weights.device, dtype=weights.dtype)
+        else:
+            w = load_hf_weights(cfg, weights.reader, tp.size, tp.rank, device=weights.device, dtype=weights.dtype)
+        self.model = create_model(cfg, w, tp)
         self.config = cfg
         self.block_size = block_size
         self.max_blocks = max_blocks
@@ -247,5 +251,10 @@ class LlamaForCausalLM(_FamilyLM):
     model_type = "llama"
 
 
+class TimisunForCausalLM(_FamilyLM):
+    """Per-layer design: latent attention + mixture of experts over an fp32 residual (models/layered.py)."""
+    model_type = "timisun"
+
+
 MODEL_REGISTRY = {c.model_type: c for c in (GPT2LMHeadModel, GPTJForCausalLM, GPTBigCodeForCausalLM,
-                                            LlamaForCausalLM)}
+                                            LlamaForCausalLM, TimisunForCausalLM)}

@@ -172,4 +172,5 @@ latent_attn = _route("latent_attn")
 latent_qa_dtype = _route("latent_qa_dtype")
 glu_clamp = _route("glu_clamp")
 moe_route = _route("moe_route")
+moe_router = _route("moe_router")
 moe_experts = _route("moe_experts")

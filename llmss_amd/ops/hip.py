@@ -1005,6 +1005,30 @@ def moe_route(z, corr, top):
     return idx, wts
 
 
+ROUTER_FUSED_MAX_ROWS = 1024  # steps of at most this many tokens compute logits and routing in one launch
+
+
+def moe_router(h, router, corr, top):
+    """(idx [T, top] int32, wts [T, top] fp32) from the layer input: fp32 router logits, then moe_route. Few rows (a
+    decode step): one fused launch; a prompt: the matrix-core GEMM with fp32 output, then moe_route."""
+    T, K = h.shape
+    E = router.shape[0]
+    if T > ROUTER_FUSED_MAX_ROWS:
+        return moe_route(linear_f(h, router, torch.float32), corr, top)
+    _rows(h, "h")
+    _check(router.dtype == h.dtype and router.is_contiguous() and router.shape == (E, K) and router.is_cuda,
+           "router [E, K] in h's storage type")
+    _check(1 <= top <= E and E <= 4096, "1 <= top <= experts <= 4096")
+    if corr is not None:
+        _check(corr.dtype == torch.float32 and corr.is_contiguous() and corr.numel() == E and corr.is_cuda,
+               "correction fp32 [E]")
+    idx = torch.empty(T, top, dtype=torch.int32, device=h.device)
+    wts = torch.empty(T, top, dtype=torch.float32, device=h.device)
+    lib().moe_router(h.data_ptr(), h.stride(0), router.data_ptr(), _ptr(corr), idx.data_ptr(), wts.data_ptr(), T, E, K,
+                     top, _dt(h, "h"), _stream())
+    return idx, wts
+
+
 def moe_experts(h, idx, wts, gate, up, down, limit, alpha, shared=None, combine=True):
     """``combine=False``: leave the weighting and summing to resid_add_norm (returns a :class:`MoEPending`)."""
     T, K = h.shape

@@ -555,6 +555,11 @@ def moe_route(z: torch.Tensor, corr: Optional[torch.Tensor], top: int):
     return idx.to(torch.int32), w
 
 
+def moe_router(h: torch.Tensor, router: torch.Tensor, corr: Optional[torch.Tensor], top: int):
+    """Router logits in fp32 from the layer input, then :func:`moe_route`."""
+    return moe_route(linear_f(h, router, torch.float32), corr, top)
+
+
 def moe_experts(h: torch.Tensor, idx: torch.Tensor, wts: torch.Tensor, gate: torch.Tensor, up: torch.Tensor,
                 down: torch.Tensor, limit: float, alpha: float, shared: Optional[torch.Tensor] = None,
                 combine: bool = True) -> torch.Tensor:

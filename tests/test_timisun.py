@@ -307,3 +307,19 @@ def test_trace_runner_replays_steps_on_the_cpu_path(cases, tmp_path):
     g2 = torch.from_numpy(np.fromfile(tmp_path / "2.f32", dtype="<f4").reshape(2, c.V))
     c.close(g0, c.ref(t)[[0, 8]], "step 0")
     c.close(g2, torch.stack([c.ref(t)[20], c.ref(t[:3])[2]]), "step 2")
+
+
+def test_registry_facade_runs_the_design(cases):
+    """MODEL_REGISTRY["timisun"](config, weights): HF-style calls with a growing paged past."""
+    from llmss_amd.models.registry import MODEL_REGISTRY, Weights
+    from llmss_amd.utils.checkpoint import weight_files
+
+    c = cases("mixed", "cpu", "float32")
+    cfg = ModelConfig.from_pretrained(c.path)
+    lm = MODEL_REGISTRY[cfg.model_type](cfg, Weights(weight_files(c.path), "cpu", torch.float32), max_blocks=16)
+    t = toks(21, c.V, 60)
+    out = lm(torch.tensor([t[:13]]), use_cache=True)
+    c.close(out.logits[0], c.ref(t[:13]), "prompt through the facade")
+    out2 = lm(torch.tensor([t[13:]]), past_key_values=out.past_key_values, use_cache=True)
+    c.close(out2.logits[0], c.ref(t)[13:], "continuation through the facade")
+    lm.release(out2.past_key_values)

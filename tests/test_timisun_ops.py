@@ -141,6 +141,9 @@ def test_mixture_of_experts(device, dtype, T, E, top, F, shared):
     idx, wts = ops.moe_route(z, sd["correction"].to(device, torch.float32), top)
     ci, cw = oracle.route(h, sd["router"], sd["correction"], top)
     assert torch.equal(idx.cpu().long().sort(-1).values, ci.sort(-1).values)
+    idx2, wts2 = ops.moe_router(hd, d(sd["router"]), sd["correction"].to(device, torch.float32), top)  # fused launch
+    assert torch.equal(idx2.cpu().long().sort(-1).values, ci.sort(-1).values)
+    assert rel(wts2.sort(-1).values, cw.sort(-1).values) < (1e-5 if dtype == torch.float32 else 1e-3)
     assert rel(wts.sum(-1), torch.ones(T, dtype=torch.double)) < 1e-5
     sh = None
     if shared:
