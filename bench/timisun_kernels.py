@@ -97,12 +97,14 @@ def main():
         # ---------------- experts vs dense gated MLP
         router, corr = rn(E, W, std=W ** -0.5), rn(E, dt=torch.float32, std=0.1)
         gate, up, down = rn(E, F, W, std=W ** -0.5), rn(E, F, W, std=W ** -0.5), rn(E, W, F, std=F ** -0.5)
-        z = ops.linear_f(h, router, torch.float32)
-        idx, wts = ops.moe_route(z, corr, top)
-        t = timed(lambda: ops.moe_route(ops.linear_f(h, router, torch.float32), corr, top))
+        t = timed(lambda: ops.moe_router(h, router, corr, top))
         add("router logits + route", phase, t)
+        # every token draws its experts uniformly, so the grouped GEMMs see balanced groups and, in a decode step,
+        # touch the experts a served batch would
+        idx = torch.rand(M, E, device=dev, generator=g).topk(top, dim=-1).indices.to(torch.int32).contiguous()
+        wts = torch.full((M, top), 1.0 / top, dtype=torch.float32, device=dev)
         t = timed(lambda: ops.moe_experts(h, idx, wts, gate, up, down, 7.0, 1.702, combine=False))
-        touched = min(E, M * top)
+        touched = int(idx.unique().numel())
         add("experts: group + gate_up + down (gemm_tile grouped)", phase, t, flops=6.0 * M * top * F * W,
             bytes_=touched * 3 * F * W * 2 + M * top * (F * 2 * 2 + W * 4) + M * W * 2)
         wu = ops.glu_interleave(rn(Fd, W, std=W ** -0.5), rn(Fd, W, std=W ** -0.5), 0)

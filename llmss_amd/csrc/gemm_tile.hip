@@ -223,8 +223,10 @@ void launch_moe_gate_up_tile(const void* h, int64_t ldh, const void* wg, const v
   a.N = F; a.K = K; a.sAm = ldh; a.sBb = (int64_t)F * K; a.sBn = K; a.sCm = F;
   a.meta = (const int*)meta; a.order = (const int*)order; a.E = E; a.maxt = maxt; a.top = top;
   a.limit = limit; a.alpha = alpha;
-  dim3 g((F + tile_rows - 1) / tile_rows, maxt);
-  if (tile_rows == 128) gemm_tile_kernel<GT_GATE_UP, bf16_t, 128, 128><<<g, 256, 0, st>>>(a);
+  // 128-row tiles are 64 columns wide here: with two accumulator sets (gate and up) a 128x128 tile leaves one
+  // workgroup per CU; at 128x64 two to three fit and hide each other's staging
+  dim3 g((F + 63) / 64, maxt);
+  if (tile_rows == 128) gemm_tile_kernel<GT_GATE_UP, bf16_t, 128, 64><<<g, 256, 0, st>>>(a);
   else gemm_tile_kernel<GT_GATE_UP, bf16_t, 64, 64><<<g, 256, 0, st>>>(a);
   HIP_CHECK_LAUNCH();
 }
