@@ -81,18 +81,18 @@ void launch_moe_route(const void* z, const void* corr, void* idx, void* wts, int
   HIP_CHECK_LAUNCH();
 }
 
-// Router logits and routing in one launch, for steps of few tokens (a decode step): one workgroup per token, its four
-// waves share the experts' dot products z_e = h . W_r[e] (fp32 accumulation over lanes), then the token is routed
+// Router logits and routing in one launch, for steps of few tokens (a decode step): one workgroup per token, its waves
+// share the experts' dot products z_e = h . W_r[e] (fp32 accumulation over lanes), then the token is routed
 // as moe_route_kernel does. A prompt's thousands of tokens take the matrix-core GEMM and moe_route instead.
 template <typename T>
-__global__ __launch_bounds__(256) void moe_router_kernel(const T* __restrict__ h, int64_t ldh, const T* __restrict__ wr,
+__global__ __launch_bounds__(1024) void moe_router_kernel(const T* __restrict__ h, int64_t ldh, const T* __restrict__ wr,
                                                          const float* __restrict__ corr, int* __restrict__ idx,
                                                          float* __restrict__ wts, int E, int K, int top, bool vec) {
   extern __shared__ float sc[];  // [E] scores, [E] choice values
   float* ch = sc + E;
-  const int t = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+  const int t = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wv = tid >> 6, nw = blockDim.x >> 6;
   const T* x = h + (int64_t)t * ldh;
-  for (int e = wv; e < E; e += 4) {
+  for (int e = wv; e < E; e += nw) {
     const T* w = wr + (int64_t)e * K;
     float acc = 0.f;
     if (vec) {  // K % 8 == 0, rows 16-byte aligned (bf16) - eight elements per lane and access
@@ -143,7 +143,7 @@ __global__ __launch_bounds__(256) void moe_router_kernel(const T* __restrict__ h
     __syncthreads();
   }
   const float inv = 1.f / (sum + 1e-20f);
-  for (int j = tid; j < top; j += 256) wts[(int64_t)t * top + j] *= inv;
+  for (int j = tid; j < top; j += blockDim.x) wts[(int64_t)t * top + j] *= inv;
 }
 
 void launch_moe_router(const void* h, int64_t ldh, const void* wr, const void* corr, void* idx, void* wts, int T_,
@@ -152,7 +152,8 @@ void launch_moe_router(const void* h, int64_t ldh, const void* wr, const void* c
   if (top > E || top <= 0) throw std::runtime_error("moe_router: top must be in [1, experts]");
   const int es = dt == 0 ? 2 : 4;
   const bool vec = K % 8 == 0 && ((uintptr_t)h % 16) == 0 && ((uintptr_t)wr % 16) == 0 && (ldh * es) % 16 == 0;
-  DISPATCH_T(dt, T, (moe_router_kernel<T><<<T_, 256, 2 * E * sizeof(float), st>>>(
+  const int threads = E >= 16 ? 1024 : (E >= 8 ? 512 : 256);  // a wave per expert up to 16 waves
+  DISPATCH_T(dt, T, (moe_router_kernel<T><<<T_, threads, 2 * E * sizeof(float), st>>>(
                         (const T*)h, ldh, (const T*)wr, (const float*)corr, (int*)idx, (float*)wts, E, K, top, vec)));
   HIP_CHECK_LAUNCH();
 }

@@ -52,9 +52,20 @@ class LatentAttention:
         if W.own_kv:
             ops.latent_norm_cache(qc, H * dim, R, W.kv_norm, model.cfg.norm_eps, cache, inp.slots)
         qa = ops.head_absorb(qc, W.uk_t, ops.latent_qa_dtype(cache))
-        o = ops.latent_attn(qa, cache, inp.block_tables, cu, inp.ctx_lens, spec.window, spec.scale,
-                            max_qlen=1 if inp.kind == "decode" else max(1, inp.max_seqlen),
-                            max_ctx=inp.max_ctx if inp.kind == "decode" else 0)
+        nd = inp.num_decode if inp.kind == "extend" else 0
+        if nd and nd < qa.shape[0]:
+            # mixed step: the single-token rows take the decode form of the kernel (their keys split over
+            # workgroups), the portions the prompt form - as DecoderLM sends its decode rows to the decode kernel
+            o = torch.cat([
+                ops.latent_attn(qa[:nd], cache, inp.block_tables[:nd], model.decode_cu(nd, qa.device),
+                                inp.ctx_lens[:nd], spec.window, spec.scale, max_qlen=1, max_ctx=inp.max_ctx),
+                ops.latent_attn(qa[nd:], cache, inp.block_tables[nd:], inp.cu_seqlens, inp.ctx_lens[nd:],
+                                spec.window, spec.scale, max_qlen=max(1, inp.max_seqlen))])
+        else:
+            single = inp.kind == "decode" or (nd and nd == qa.shape[0])
+            o = ops.latent_attn(qa, cache, inp.block_tables, cu, inp.ctx_lens, spec.window, spec.scale,
+                                max_qlen=1 if single else max(1, inp.max_seqlen),
+                                max_ctx=inp.max_ctx if single else 0)
         return ops.linear_f(ops.head_expand(o, W.uv, dt), W.o, dt)
 
 
