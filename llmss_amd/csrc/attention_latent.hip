@@ -165,7 +165,8 @@ static void latent_attn_t(const void* qa, int64_t ldq, const void* cache, const 
   else if (nr <= 2) LAUNCH_LA(2);
   else if (nr <= 4) LAUNCH_LA(4);
   else if (nr <= 8) LAUNCH_LA(8);
-  else throw std::runtime_error("latent attention: latent rank above 512");
+  else if (nr <= 16) LAUNCH_LA(16);
+  else throw std::runtime_error("latent attention: latent rank above 1024");
 #undef LAUNCH_LA
 }
 

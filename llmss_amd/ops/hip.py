@@ -973,7 +973,7 @@ def latent_attn(qa, cache, block_tables, cu_q, ctx_lens, window, scale, max_qlen
                           window=window, key_split=split)
         return out.view(T, H, R)
     _check(qa.dtype == torch.float32, "qa fp32")
-    _check(R <= 512, "latent rank above 512")
+    _check(R <= 1024, "latent rank above 1024")
     out = torch.empty(T, H, R, dtype=torch.float32, device=qa.device)
     lib().latent_attn(qa.data_ptr(), H * R, cache.data_ptr(), block_tables.data_ptr(), block_tables.shape[1],
                       cu_q.data_ptr(), ctx_lens.data_ptr(), out.data_ptr(), H * R, T, B, H, R, cache.shape[1],

@@ -100,6 +100,19 @@ def test_latent_attention_standout_key(device, dtype, window, back, R):
 
 
 @pytest.mark.parametrize("device,dtype", RUNS)
+@pytest.mark.parametrize("R,window", [(600, 0), (520, 17), (130, 5)])
+def test_latent_attention_ranks_beyond_the_matrix_core_kernel(device, dtype, R, window):
+    heads, dim, vdim, W, block, T = 2, 8, 8, 24, 16, 37
+    h, c = rnd(T, W, seed=30), rnd(T, R, seed=31, std=0.5)
+    wq, wuk = rnd(heads * dim, W, seed=32, std=W ** -0.5), rnd(heads * dim, R, seed=33, std=R ** -0.5)
+    wuv, wo = rnd(heads * vdim, R, seed=34, std=R ** -0.5), rnd(W, heads * vdim, seed=35, std=0.2)
+    want = oracle.latent_attention(h, c, wq, wuk, wuv, wo, heads, dim, vdim, 0.4, window)
+    for portions in ([T], [T - 3, 2, 1]):
+        got = run_attention(device, dtype, h, c, wq, wuk, wuv, wo, heads, dim, vdim, 0.4, window, block, portions)
+        assert rel(got, want) < tol(dtype, f32=5e-5, bf16=3e-2), (portions, rel(got, want))
+
+
+@pytest.mark.parametrize("device,dtype", RUNS)
 def test_latent_rows_are_normed_into_their_slots(device, dtype):
     T, R, off, block = 7, 24, 16, 4
     src, w = rnd(T, off + R + 8, seed=12, std=3.0), rnd(R, seed=13)
