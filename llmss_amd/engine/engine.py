@@ -219,7 +219,7 @@ class LLMEngine:
         if autotune is None:
             autotune = os.environ.get("LLMSS_AUTOTUNE", "1") != "0"
         self.tuned = {}
-        if self.is_gpu and autotune and self._uniform:  # per-shape GEMM plans for every decode bucket (ops/autotune.py)
+        if self.is_gpu and autotune:  # per-shape GEMM plans for every decode bucket (ops/autotune.py)
             from ..ops.autotune import tune_model
 
             self.tuned = tune_model(model, self.decode_batch_sizes())

@@ -128,6 +128,29 @@ class LayeredLM:
     def overlap_split(self, B: int) -> int:
         return 0
 
+    def gemm_shapes(self):
+        """The dense projections that run on the autotuned MFMA GEMM (ops.linear_f -> ops/hip.py linear), one entry
+        per distinct [N, K]: query | latent, output, the shared expert's two products and the head. The engine's
+        autotuner times plans for them per decode bucket (ops/autotune.py)."""
+        from ..ops.autotune import GemmShape
+
+        if self.dtype != torch.bfloat16:
+            return {}
+        out = {}
+
+        def put(name, w):
+            N, K = w.shape
+            if K % 16 == 0 and N % 8 == 0 and (N, K) not in {(s.N, s.K) for s in out.values()}:
+                out[f"{name}_{N}x{K}"] = GemmShape(N, K)
+        for L in self.w.layers:
+            put("qc", L.mix.qc)
+            put("o", L.mix.o)
+            if L.mlp is not None and L.mlp.shared_gu is not None:
+                put("shared_gu", L.mlp.shared_gu)
+                put("shared_down", L.mlp.shared_down)
+        put("head", self.w.head.w)
+        return out
+
     # --------------------------------------------------------------------------------- cache
     def _cache_rows(self) -> List[Optional[int]]:
         return [MIXERS[s.mixer.kind].cache_row(s.mixer) for s in self.cfg.layer_specs]

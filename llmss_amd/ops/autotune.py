@@ -203,7 +203,10 @@ def tune_shape(M: int, shape: GemmShape, device, weight_budget: int = 600 << 20,
 
 
 def model_shapes(model) -> Dict[str, GemmShape]:
-    """The per-layer projections of a DecoderLM (layer 0 is representative) + the LM head."""
+    """The per-layer projections of a DecoderLM (layer 0 is representative) + the LM head; a model that describes
+    its own dense projections (``gemm_shapes()``: per-layer designs, whose layers differ) is asked instead."""
+    if hasattr(model, "gemm_shapes"):
+        return model.gemm_shapes()
     L = model.w.layers[0]
     fuse = model.tp.size == 1 and not model.cfg.parallel_block
     act = model.act if not L.up.glu else "none"
@@ -363,6 +366,10 @@ def tune_model(model, ms: Sequence[int], native=None) -> Dict[Tuple[str, int], T
             if nt:
                 lib.gemm_tuned_set(M, shp.N, shp.K, shp.glu, int(shp.fp8), nt, s)
             res[(name, M)] = done[key]
+    if hasattr(model, "gemm_shapes"):  # no fused-QKV projection to tune
+        torch.cuda.synchronize(dev)
+        log.info("autotuned %d GEMM shapes in %.1fs", len(res), time.perf_counter() - t0)
+        return res
     # the fused QKV epilogue is a candidate wherever it applies (tune_qkv_epilogue decides per bucket)
     key = ("qkv_epi", tuple(sorted(set(int(m) for m in ms))), model_shapes(model)["qkv"], str(dev),
            model.cfg.head_dim, model.cfg.rotary_dim, model.cfg.rope_style, model.cfg.position)

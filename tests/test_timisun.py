@@ -323,3 +323,20 @@ def test_registry_facade_runs_the_design(cases):
     out2 = lm(torch.tensor([t[13:]]), past_key_values=out.past_key_values, use_cache=True)
     c.close(out2.logits[0], c.ref(t)[13:], "continuation through the facade")
     lm.release(out2.past_key_values)
+
+
+@gpu
+def test_engine_autotunes_the_dense_projections_and_still_decodes_right(cases):
+    """With the GEMM autotuner on (the serving default) the plans of the query | latent, output, shared-expert and
+    head products are timed per decode bucket; greedy decoding through the captured graphs stays right."""
+    c = cases("wide", "cuda", "bfloat16")
+    assert c.model.gemm_shapes()
+    eng = LLMEngine(c.model, max_num_seqs=2, block_size=16, num_blocks=16, max_model_len=96, max_batched_tokens=64)
+    assert eng.tuned and eng.graphs
+    p = toks(9, c.V, 70)
+    out = eng.generate([p], SamplingParams(max_new_tokens=6, is_greedy=True, ignore_eos=True))[0]
+    want = oracle.greedy(c.cfg, c.sd, p, 6)
+    k = next((i for i, (x, y) in enumerate(zip(out, want)) if x != y), None)
+    if k is not None:
+        lg = oracle.forward(c.cfg, c.sd, p + want[:k])[0][-1]
+        assert float(lg[want[k]] - lg[out[k]]) < 0.05 * float(lg.std())
