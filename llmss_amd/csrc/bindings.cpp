@@ -110,6 +110,33 @@ void launch_moe_combine(const void* y, const void* place, const void* wts, const
 void launch_glu_clamp(const void* gu, int64_t ldg, void* out, int64_t ldo, int T_, int F, float limit, float alpha,
                       int dt, hipStream_t st);
 
+// residual streams, causal convolutions with a per-sequence tail, matrix-state recurrences, sink attention
+void launch_embed_streams(const void* ids, const void* positions, const void* table, const void* ptab, void* x, int S,
+                          int T_, int W, int vocab, int npos, int dt, hipStream_t st);
+void launch_stream_add_norm(void* x, const void* y, int64_t ldy, const void* mix, const void* outw, float c,
+                            const void* inw, const void* w, float eps, int rms, void* h, int64_t ldh, int S, int T_,
+                            int W, int dt, int h_f32, hipStream_t st);
+void launch_causal_conv(const void* in, int64_t ldi, const void* w, void* state, const void* cu, const void* ctx,
+                        const void* sslots, void* out, int64_t ldo, int T_, int B, int C, int taps, int res, int silu,
+                        int di, int dw, int dout, hipStream_t st);
+void launch_gated_group_norm(const void* o, int64_t ldo, const void* gate, int64_t ldg, const void* w, float eps,
+                             int act, float c, void* out, int64_t ldout, int T_, int groups, int n, int dt,
+                             hipStream_t st);
+void launch_glu_act(const void* gu, int64_t ldg, void* out, int64_t ldo, int T_, int F, int act, int dt,
+                    hipStream_t st);
+void launch_recurrence(int mode, const void* q, const void* k, const void* v, int64_t ldq, int64_t ldk, int64_t ldv,
+                       const void* ab, int64_t ldab, int off_a, int off_b, const void* decay, const void* dt_bias,
+                       void* state, const void* cu, const void* ctx, const void* sslots, void* out, int64_t ldo, int B,
+                       int H, int G, int dim, int vdim, int silu_in, int dq, int dp, hipStream_t st);
+void launch_rope_bias_cache(const void* proj, int64_t ldp, int off_q, int off_k, int off_v, const void* bias,
+                            const void* positions, const void* cs, int npos, int rot, void* qout, void* kc, void* vc,
+                            const void* slots, int T_, int H, int G, int dim, int vdim, int dt, hipStream_t st);
+void launch_sink_attn(const void* q, const void* kc, const void* vc, const void* bt, int maxb, const void* cu,
+                      const void* ctx, void* out, int T_, int B, int H, int G, int dim, int vdim, int bs, float scale,
+                      float cap, int all, int dt, hipStream_t st);
+void launch_talk_mix(const void* O, const void* talk, float c, void* y, int64_t ldy, int T_, int H, int G, int vdim,
+                     int dt, hipStream_t st);
+
 void register_runtime(py::module_& m);  // host-side C++ runtime (runtime.cpp)
 void register_comm(py::module_& m);     // RCCL communicator (comm.cpp)
 void register_ctrl(py::module_& m);     // shared-memory control ring (ctrl.cpp)
@@ -308,6 +335,50 @@ PYBIND11_MODULE(_C, m) {
   });
   m.def("glu_clamp", [](uintptr_t gu, int64_t ldg, uintptr_t out, int64_t ldo, int T, int F, float limit, float alpha,
                         int dt, uintptr_t st) { launch_glu_clamp(CP(gu), ldg, P(out), ldo, T, F, limit, alpha, dt, S(st)); });
+  m.def("embed_streams", [](uintptr_t ids, uintptr_t pos, uintptr_t table, uintptr_t ptab, uintptr_t x, int Sn, int T,
+                            int W, int V, int npos, int dt, uintptr_t st) {
+    launch_embed_streams(CP(ids), CP(pos), CP(table), CP(ptab), P(x), Sn, T, W, V, npos, dt, S(st));
+  });
+  m.def("stream_add_norm", [](uintptr_t x, uintptr_t y, int64_t ldy, uintptr_t mix, uintptr_t outw, float c,
+                              uintptr_t inw, uintptr_t w, float eps, int rms, uintptr_t h, int64_t ldh, int Sn, int T,
+                              int W, int dt, int h_f32, uintptr_t st) {
+    launch_stream_add_norm(P(x), CP(y), ldy, CP(mix), CP(outw), c, CP(inw), CP(w), eps, rms, P(h), ldh, Sn, T, W, dt,
+                           h_f32, S(st));
+  });
+  m.def("causal_conv", [](uintptr_t in, int64_t ldi, uintptr_t w, uintptr_t state, uintptr_t cu, uintptr_t ctx,
+                          uintptr_t ss, uintptr_t out, int64_t ldo, int T, int B, int C, int taps, int res, int silu,
+                          int di, int dw, int dout, uintptr_t st) {
+    launch_causal_conv(CP(in), ldi, CP(w), P(state), CP(cu), CP(ctx), CP(ss), P(out), ldo, T, B, C, taps, res, silu,
+                       di, dw, dout, S(st));
+  });
+  m.def("gated_group_norm", [](uintptr_t o, int64_t ldo, uintptr_t gate, int64_t ldg, uintptr_t w, float eps, int act,
+                               float c, uintptr_t out, int64_t ldout, int T, int groups, int n, int dt, uintptr_t st) {
+    launch_gated_group_norm(CP(o), ldo, CP(gate), ldg, CP(w), eps, act, c, P(out), ldout, T, groups, n, dt, S(st));
+  });
+  m.def("glu_act", [](uintptr_t gu, int64_t ldg, uintptr_t out, int64_t ldo, int T, int F, int act, int dt,
+                      uintptr_t st) { launch_glu_act(CP(gu), ldg, P(out), ldo, T, F, act, dt, S(st)); });
+  m.def("recurrence", [](int mode, uintptr_t q, uintptr_t k, uintptr_t v, int64_t ldq, int64_t ldk, int64_t ldv,
+                         uintptr_t ab, int64_t ldab, int off_a, int off_b, uintptr_t decay, uintptr_t dtb,
+                         uintptr_t state, uintptr_t cu, uintptr_t ctx, uintptr_t ss, uintptr_t out, int64_t ldo, int B,
+                         int H, int G, int dim, int vdim, int silu_in, int dq, int dp, uintptr_t st) {
+    launch_recurrence(mode, CP(q), CP(k), CP(v), ldq, ldk, ldv, CP(ab), ldab, off_a, off_b, CP(decay), CP(dtb),
+                      P(state), CP(cu), CP(ctx), CP(ss), P(out), ldo, B, H, G, dim, vdim, silu_in, dq, dp, S(st));
+  });
+  m.def("rope_bias_cache", [](uintptr_t proj, int64_t ldp, int off_q, int off_k, int off_v, uintptr_t bias,
+                              uintptr_t pos, uintptr_t cs, int npos, int rot, uintptr_t qout, uintptr_t kc,
+                              uintptr_t vc, uintptr_t slots, int T, int H, int G, int dim, int vdim, int dt,
+                              uintptr_t st) {
+    launch_rope_bias_cache(CP(proj), ldp, off_q, off_k, off_v, CP(bias), CP(pos), CP(cs), npos, rot, P(qout), P(kc),
+                           P(vc), CP(slots), T, H, G, dim, vdim, dt, S(st));
+  });
+  m.def("sink_attn", [](uintptr_t q, uintptr_t kc, uintptr_t vc, uintptr_t bt, int maxb, uintptr_t cu, uintptr_t ctx,
+                        uintptr_t out, int T, int B, int H, int G, int dim, int vdim, int bs, float scale, float cap,
+                        int all, int dt, uintptr_t st) {
+    launch_sink_attn(CP(q), CP(kc), CP(vc), CP(bt), maxb, CP(cu), CP(ctx), P(out), T, B, H, G, dim, vdim, bs, scale,
+                     cap, all, dt, S(st));
+  });
+  m.def("talk_mix", [](uintptr_t O, uintptr_t talk, float c, uintptr_t y, int64_t ldy, int T, int H, int G, int vdim,
+                       int dt, uintptr_t st) { launch_talk_mix(CP(O), CP(talk), c, P(y), ldy, T, H, G, vdim, dt, S(st)); });
   register_runtime(m);
   register_comm(m);
   register_ctrl(m);

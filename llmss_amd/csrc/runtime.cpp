@@ -104,6 +104,7 @@ struct SeqState {
   int status;  // 0 waiting, 1 running, 2 finished
   int64_t order;
   int preemptions = 0;
+  int state_slot = -1;  // running sequences: index of the per-sequence state slot (recurrent state, convolution tails)
 };
 
 struct StepBatch {
@@ -116,6 +117,7 @@ struct StepBatch {
   std::vector<int64_t> positions;
   std::vector<int64_t> slots;
   std::vector<int> block_table;  // [B, max_blocks] padded with 0
+  std::vector<int> state_slots;  // per sequence: its state slot in [0, max_num_seqs)
   int max_blocks = 0;
   std::vector<int64_t> preempted;
 };
@@ -139,6 +141,7 @@ class Scheduler {
         max_len_(max_model_len),
         chunk_(prefill_chunk) {
     max_blocks_per_seq_ = (max_model_len + block_size - 1) / block_size;
+    for (int i = max_num_seqs - 1; i >= 0; --i) free_state_.push_back(i);
     if (max_batched_tokens <= 0) throw std::invalid_argument("Scheduler: max_batched_tokens must be > 0");
   }
 
@@ -179,6 +182,7 @@ class Scheduler {
     auto& s = it->second;
     alloc_.free_all(s.blocks);
     s.blocks.clear();
+    release_state(s);
     if (s.status == 1) running_.erase(std::remove(running_.begin(), running_.end(), id), running_.end());
     if (s.status == 0) waiting_.erase(std::remove(waiting_.begin(), waiting_.end(), id), waiting_.end());
     seqs_.erase(it);
@@ -224,6 +228,7 @@ class Scheduler {
           SeqState s{ids[i], 0, max_len_, 0, 0, {}, 1, counter_++};
           it = seqs_.emplace(ids[i], s).first;
           running_.push_back(ids[i]);
+          take_state(it->second);
         }
         auto& s = it->second;
         s.num_tokens += counts[i];
@@ -318,6 +323,7 @@ class Scheduler {
       s.status = 1;
       waiting_.pop_front();
       running_.push_back(s.id);
+      take_state(s);
       emit(b, s, q);
       budget -= q;
     }
@@ -352,6 +358,7 @@ class Scheduler {
     return s.blocks[(n_tokens - 1) / bs_];
   }
   int num_tokens(int64_t id) { return get(id).num_tokens; }
+  int state_slot(int64_t id) { return get(id).state_slot; }
   int num_computed(int64_t id) { return get(id).num_computed; }
   std::vector<int> blocks(int64_t id) { return get(id).blocks; }
   bool contains(int64_t id) const { return seqs_.count(id) > 0; }
@@ -378,9 +385,24 @@ class Scheduler {
     for (int i = 0; i < need; ++i) s.blocks.push_back(alloc_.allocate());
     return true;
   }
+  // State slots: one per running sequence, handed out on admission and given back on finish / preemption. A
+  // sequence whose portion starts at position 0 starts from an empty state whatever its slot held, so a slot is
+  // never cleared.
+  void take_state(SeqState& s) {
+    if (s.state_slot >= 0) return;
+    if (free_state_.empty()) throw std::runtime_error("Scheduler: no free state slot");
+    s.state_slot = free_state_.back();
+    free_state_.pop_back();
+  }
+  void release_state(SeqState& s) {
+    if (s.state_slot < 0) return;
+    free_state_.push_back(s.state_slot);
+    s.state_slot = -1;
+  }
   void emit(StepBatch& b, SeqState& s, int q) {
     const int p0 = s.num_computed;
     b.ids.push_back(s.id);
+    b.state_slots.push_back(s.state_slot);
     b.query_lens.push_back(q);
     b.ctx_lens.push_back(p0 + q);
     for (int p = p0; p < p0 + q; ++p) {
@@ -397,6 +419,7 @@ class Scheduler {
     s.num_computed = 0;
     s.status = 0;
     s.preemptions++;
+    release_state(s);
     running_.erase(std::remove(running_.begin(), running_.end(), id), running_.end());
     waiting_.push_front(id);
   }
@@ -411,6 +434,7 @@ class Scheduler {
   }
 
   BlockAllocator alloc_;
+  std::vector<int> free_state_;
   int bs_, max_seqs_, max_tokens_, max_len_, max_blocks_per_seq_, chunk_;
   std::unordered_map<int64_t, SeqState> seqs_;
   std::deque<int64_t> waiting_;
@@ -758,6 +782,7 @@ void register_runtime(py::module_& m) {
                                a.resize({B, (ssize_t)b.max_blocks});
                                return a;
                              })
+      .def_property_readonly("state_slots", [](const StepBatch& b) { return to_np(b.state_slots); })
       .def_property_readonly("preempted", [](const StepBatch& b) { return to_np(b.preempted); });
 
   py::class_<Scheduler>(m, "Scheduler")
@@ -784,6 +809,7 @@ void register_runtime(py::module_& m) {
       .def("max_blocks_per_seq", &Scheduler::max_blocks_per_seq)
       .def("has_work", &Scheduler::has_work)
       .def("num_tokens", &Scheduler::num_tokens)
+      .def("state_slot", &Scheduler::state_slot)
       .def("reserve", &Scheduler::reserve)
       .def("blocks", &Scheduler::blocks)
       .def("contains", &Scheduler::contains);

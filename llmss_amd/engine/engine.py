@@ -92,8 +92,8 @@ class _DecodeBuffers:
         B, MB = max_b, max_blocks
         self.max_b, self.max_blocks = B, MB
         pin = torch.cuda.is_available() and device.type == "cuda"
-        self.o32 = 4 * B * 8  # ids|pos|slots|seeds (i64) | ctx|topk|bt (i32) | temp|topp (f32)
-        self.of32 = self.o32 + (2 * B + B * MB) * 4
+        self.o32 = 4 * B * 8  # ids|pos|slots|seeds (i64) | ctx|topk|state slots|bt (i32) | temp|topp (f32)
+        self.of32 = self.o32 + (3 * B + B * MB) * 4
         nbytes = self.of32 + 2 * B * 4
         self.h = [torch.zeros(nbytes, dtype=torch.uint8, pin_memory=pin) for _ in range(2)]
         self.d = torch.zeros(nbytes, dtype=torch.uint8, device=device)
@@ -103,11 +103,11 @@ class _DecodeBuffers:
         self.out = torch.zeros(max_b, dtype=torch.int64, device=device)
         self.h_out = [torch.zeros(max_b, dtype=torch.int64, pin_memory=pin) for _ in range(2)]
         self.ids, self.pos, self.slots, self.seeds = (self.d_i64[i * B:(i + 1) * B] for i in range(4))
-        self.ctx, self.topk = self.d_i32[:B], self.d_i32[B:2 * B]
-        self.bt = self.d_i32[2 * B:].view(B, max_blocks)
+        self.ctx, self.topk, self.sslots = self.d_i32[:B], self.d_i32[B:2 * B], self.d_i32[2 * B:3 * B]
+        self.bt = self.d_i32[3 * B:].view(B, max_blocks)
         self.temp, self.topp = self.d_f32[:B], self.d_f32[B:]
 
-    def fill(self, k, b_pad, ids, pos, slots, seeds, ctx, topk, bt, temp, topp):
+    def fill(self, k, b_pad, ids, pos, slots, seeds, ctx, topk, bt, temp, topp, sslots=None):
         """Stage one step's inputs in set k and copy them to the device. ``ids=None``: the input ids
         are the previous step's sampled tokens, copied on the device (same rows)."""
         n = len(pos)
@@ -124,7 +124,10 @@ class _DecodeBuffers:
         hi32[n:b_pad] = 0
         hi32[B:B + n] = topk
         hi32[B + n:B + b_pad] = 1
-        btv = hi32[2 * B:].reshape(B, MB)
+        hi32[2 * B:2 * B + b_pad] = -1  # padded rows and models without per-sequence state: no state slot
+        if sslots is not None:
+            hi32[2 * B:2 * B + n] = sslots
+        btv = hi32[3 * B:].reshape(B, MB)
         btv[:n, :bt.shape[1]] = bt
         btv[n:b_pad] = 0
         hf[:n] = temp
@@ -165,7 +168,11 @@ class LLMEngine:
         # preemption) must be identical everywhere: each rank sizes it from its own free HBM, then all
         # take the minimum
         self.num_blocks = self.tp.all_reduce_int(num_blocks or self._auto_blocks(kv_fraction), "min")
-        self.kv = model.allocate_kv_cache(self.num_blocks, block_size)
+        # models with per-sequence state (recurrent mixers, convolution tails) get one state slot per sequence the
+        # scheduler can run; the scheduler hands the slots out and the steps carry them (StepInput.state_slots)
+        self.stateful = bool(getattr(model, "needs_state", False))
+        self.kv = (model.allocate_kv_cache(self.num_blocks, block_size, num_slots=max_num_seqs) if self.stateful
+                   else model.allocate_kv_cache(self.num_blocks, block_size))
         # chunked prefill: prompts are cut to fit the per-step token budget and ride along with the
         # running decodes (prefill_chunk > 0 caps a chunk further; < 0 keeps prompts whole)
         self.prefill_chunk = int(prefill_chunk if prefill_chunk is not None else
@@ -284,6 +291,8 @@ class LLMEngine:
         if self.is_gpu:
             free, _ = torch.cuda.mem_get_info(self.device)
             budget = int(free * frac) - (4 << 30)
+            if getattr(self.model, "needs_state", False):
+                budget -= self.max_num_seqs * self.model.state_bytes_per_slot()
             n = max(64, budget // per)
             return int(min(n, want))
         return int(min(want, max(64, (2 << 30) // per)))
@@ -566,10 +575,11 @@ class LLMEngine:
             return torch.from_numpy(np.ascontiguousarray(a)).to(dev, non_blocking=True)
 
         bt, cl = d(batch.block_table.astype(np.int32)), d(ctx.astype(np.int32))
+        ss = d(batch.state_slots.astype(np.int32)) if self.stateful else None
         li = d(np.asarray(last_idx, dtype=np.int64)) if last_idx is not None else None
         if nd == len(qlens):  # single tokens only
             return StepInput(kind="decode", input_ids=d(ids), positions=d(batch.positions), slots=d(batch.slots),
-                             block_tables=bt, ctx_lens=cl, max_ctx=self.max_model_len, last_idx=li)
+                             block_tables=bt, ctx_lens=cl, max_ctx=self.max_model_len, last_idx=li, state_slots=ss)
         ends = np.cumsum(qlens)
         cu = np.zeros(len(qlens) - nd + 1, dtype=np.int32)
         cu[1:] = ends[nd:] - (ends[nd - 1] if nd else 0)
@@ -578,7 +588,7 @@ class LLMEngine:
         return StepInput(
             kind=kind, input_ids=d(ids), positions=d(batch.positions), slots=d(batch.slots), cu_seqlens=d(cu),
             max_seqlen=int(qlens[nd:].max()), last_idx=li, block_tables=bt, ctx_lens=cl, max_ctx=self.max_model_len,
-            num_decode=nd, has_prefix=has_prefix, cu_host=cu if kind == "prefill" else None)
+            num_decode=nd, has_prefix=has_prefix, cu_host=cu if kind == "prefill" else None, state_slots=ss)
 
     def _extend(self, batch, reqs: List[Request]) -> List[int]:
         """A step with prompt chunks: rows [0, num_decode) are decode tokens, then one chunk per
@@ -657,7 +667,7 @@ class LLMEngine:
     def _decode_forward(self, b: int, buf: _DecodeBuffers, dist: bool = False):
         inp = StepInput(kind="decode", input_ids=buf.ids[:b], positions=buf.pos[:b], slots=buf.slots[:b],
                         block_tables=buf.bt[:b], ctx_lens=buf.ctx[:b], max_ctx=self.max_model_len,
-                        decode_splits=self._splits(b))
+                        decode_splits=self._splits(b), state_slots=buf.sslots[:b] if self.stateful else None)
         self._forward_sample(inp, buf.temp[:b], buf.topk[:b], buf.topp[:b], buf.seeds[:b], out=buf.out[:b],
                              dist=dist)
 
@@ -667,7 +677,8 @@ class LLMEngine:
         inp = StepInput(kind="decode", input_ids=torch.from_numpy(ids), positions=torch.from_numpy(batch.positions),
                         slots=torch.from_numpy(batch.slots),
                         block_tables=torch.from_numpy(batch.block_table.astype(np.int32)),
-                        ctx_lens=torch.from_numpy(batch.ctx_lens.astype(np.int32)), max_ctx=self.max_model_len)
+                        ctx_lens=torch.from_numpy(batch.ctx_lens.astype(np.int32)), max_ctx=self.max_model_len,
+                        state_slots=torch.from_numpy(batch.state_slots.astype(np.int32)) if self.stateful else None)
         return self._forward_sample(inp, temp, topk, topp, seeds, dist=self._dist_ok(temp, topk)).tolist()
 
     # ------------------------------------------------------------------ pipelined GPU decode
@@ -689,7 +700,8 @@ class LLMEngine:
                  "nout": np.array([len(r.output_ids) for r in reqs], dtype=np.int64),
                  "last": np.array([r.last_id for r in reqs], dtype=np.int64)}
         c.update(ids=ids, reqs=reqs, n=len(reqs), pos=batch.positions, ctx=batch.ctx_lens.astype(np.int32),
-                 slots=batch.slots, bt=batch.block_table, keep=np.ones(len(reqs), dtype=bool))
+                 slots=batch.slots, bt=batch.block_table, keep=np.ones(len(reqs), dtype=bool),
+                 sslots=batch.state_slots.astype(np.int32))
         c["dist"] = self._dist_ok(c["temp"], c["topk"])
         return c
 
@@ -703,7 +715,7 @@ class LLMEngine:
         with self.timer.phase("decode"):
             buf.fill(k, b, None if device_ids else rec.pop("last"), rec["pos"], rec["slots"],
                      step_seeds(rec["seed"], rec["nout"]), rec["ctx"], rec["topk"], rec["bt"], rec["temp"],
-                     rec["topp"])
+                     rec["topp"], sslots=rec["sslots"] if self.stateful else None)
             key = (b, bool(rec["dist"]))
             if self._host_prof:
                 # was the GPU already idle (every earlier step done) when this step was launched?
@@ -754,6 +766,7 @@ class LLMEngine:
         rec["pos"] = nxt_pos
         rec["ctx"] = np.where(alive, cur["ctx"] + 1, 0).astype(np.int32)
         rec["slots"] = slots
+        rec["sslots"] = np.where(alive, cur["sslots"], -1).astype(np.int32)  # a stopped row leaves its state alone
         rec["nout"] = cur["nout"] + 1
         rec["keep"] = alive
         if dead.any():
@@ -812,6 +825,7 @@ class LLMEngine:
         buf.slots.fill_(-1)
         buf.d_i32.zero_()
         buf.topk.fill_(1)
+        buf.sslots.fill_(-1)
         buf.d_f32.zero_()
         modes = self._decode_modes()
         # warm-up passes (lazy allocations, first launches). Native RCCL: with real collectives, so each

@@ -22,6 +22,7 @@ Families (``MODEL_REGISTRY`` keys, reference ``custom_modeling/__init__.py:4-7``
 from __future__ import annotations
 
 import json
+import math
 import os
 from dataclasses import asdict, dataclass, field, replace
 from typing import Any, Dict, List, Optional
@@ -61,9 +62,77 @@ class MoESpec:
 
 
 @dataclass
+class RotarySpec:
+    """Rotary positions on the first ``dims`` dimensions of a head, dimension i paired with i + dims / 2, frequency
+    base^(-2 i / dims); ``scaling`` = (factor, original length, fast turns, slow turns) blends the frequencies
+    between the two turn counts towards f / factor and scales cos and sin by 0.1 ln(factor) + 1."""
+    dims: int
+    base: float
+    scaling: Optional[tuple] = None
+
+
+@dataclass
+class SinkAttnSpec:
+    """Softmax attention over a paged key/value cache: ``heads`` query heads on ``kv_heads`` key/value heads, key
+    size ``dim``, value size ``vdim``; scores times ``scale``, soft-capped when ``softcap`` > 0; one unit added to
+    the softmax denominator (a sink); ``talk``: the heads' weights are mixed by an [heads, heads] matrix; ``bias``:
+    the q / k / v projections have biases."""
+    heads: int
+    kv_heads: int
+    dim: int
+    vdim: int
+    scale: float
+    softcap: float = 0.0
+    rot: Optional[RotarySpec] = None
+    talk: bool = False
+    bias: bool = False
+    kind: str = "sink_attention"
+
+
+@dataclass
+class DeltaSpec:
+    """Gated delta rule: a matrix state [dim, vdim] per head, ``kv_heads`` query/key heads shared by ``heads`` value
+    heads, q / k / v through a short causal convolution of ``conv`` taps."""
+    heads: int
+    kv_heads: int
+    dim: int
+    vdim: int
+    conv: int
+    kind: str = "gated_delta"
+
+
+@dataclass
+class DecaySpec:
+    """Linear attention with a constant decay per head over a matrix state [dim, vdim]."""
+    heads: int
+    dim: int
+    vdim: int
+    decay: tuple = ()
+    kind: str = "lightning"
+
+
+@dataclass
+class ParallelMixerSpec:
+    """Two mixers reading the same input; the result is left_scale * left + right_scale * right."""
+    left: SinkAttnSpec
+    right: DeltaSpec
+    left_scale: float = 1.0
+    right_scale: float = 1.0
+    kind: str = "parallel"
+
+
+@dataclass
+class DenseMLPSpec:
+    """Gated feed-forward down(act(gate h) * (up h))."""
+    ff: int
+    act: str = "gelu_tanh"
+    kind: str = "dense"
+
+
+@dataclass
 class LayerSpec:
-    mixer: MixerSpec
-    mlp: Optional[MoESpec] = None
+    mixer: Any
+    mlp: Optional[Any] = None
 
 
 @dataclass
@@ -101,6 +170,10 @@ class ModelConfig:
     embedding_scale: float = 1.0  # the embedding row is multiplied by this
     norm_offset: float = 0.0  # norm weights are stored as (w - offset): 1.0 = stored around zero
     residual_fp32: bool = False  # the residual stream is kept and summed in fp32
+    # sequential per-layer blocks (x <- x + c * mixer(norm1(x)); x <- x + c * ffn(norm2(x))):
+    streams: int = 0  # > 0: that many residual streams with learned read / write / mix weights per sublayer
+    residual_mult: float = 1.0  # c above
+    canon_taps: int = 0  # > 0: the mixer's input h becomes h + causal_conv(h) over that many taps
 
     # ---------------------------------------------------------------- derived
     @property
@@ -121,6 +194,10 @@ class ModelConfig:
 
     def num_params(self) -> int:
         h, f, v = self.hidden_size, self.intermediate_size, self.vocab_size
+        if self.layer_specs and self.model_type == "babotar":
+            from .weights import babotar_shapes
+
+            return sum(math.prod(shp) for shp in babotar_shapes(self).values())
         if self.layer_specs:
             n = v * h + h
             for s in self.layer_specs:
@@ -147,6 +224,8 @@ class ModelConfig:
         mt = d.get("model_type")
         if mt is None and d.get("architecture") == "Timisun":
             return _timisun(cls, d)
+        if mt is None and d.get("architecture") == "Babotar":
+            return _babotar(cls, d)
         common = dict(
             bos_token_id=d.get("bos_token_id"),
             eos_token_id=_first(d.get("eos_token_id")),
@@ -255,6 +334,64 @@ def _timisun(cls, d: Dict[str, Any]) -> "ModelConfig":
     )
 
 
+def _babotar(cls, d: Dict[str, Any]) -> "ModelConfig":
+    """``{"architecture": "Babotar", "vocab", "width", "max_positions", "norm": {"eps"}, "residual_mult", "streams",
+    "canon": {"taps"}, "layers": [{"type": "lightning" | "parallel", "mixer": {...}, "mlp": {"kind": "dense", "ff"} |
+    null}]}``. A lightning mixer gives heads, dim, vdim, decay; a parallel one ``left`` (heads, kv_heads, dim, vdim,
+    scale, softcap, rot: {base, dims, scaling: {factor, original, fast, slow}}), ``right`` (heads, kv_heads, dim,
+    vdim, conv), left_scale, right_scale. Keys that a config leaves out switch their mechanism off (no streams, no
+    input convolution, no cap, no rotation, no frequency scaling); the head-mixing matrix and the q / k / v biases
+    are found by their tensors at load."""
+    specs: List[LayerSpec] = []
+    for i, L in enumerate(d["layers"]):
+        m, typ = L["mixer"], L.get("type")
+        if typ == "lightning":
+            mixer = DecaySpec(int(m["heads"]), int(m["dim"]), int(m["vdim"]), tuple(float(x) for x in m["decay"]))
+            if len(mixer.decay) != mixer.heads:
+                raise ValueError(f"Babotar layer {i}: {len(mixer.decay)} decays for {mixer.heads} heads")
+        elif typ == "parallel":
+            a, r = m["left"], m["right"]
+            rot = None
+            if a.get("rot"):
+                sc = a["rot"].get("scaling")
+                rot = RotarySpec(int(a["rot"]["dims"]), float(a["rot"]["base"]),
+                                 None if not sc else (float(sc["factor"]), float(sc["original"]), float(sc["fast"]),
+                                                      float(sc["slow"])))
+                if rot.dims % 2 or rot.dims > int(a["dim"]):
+                    raise ValueError(f"Babotar layer {i}: {rot.dims} rotary dimensions on heads of {a['dim']}")
+            left = SinkAttnSpec(int(a["heads"]), int(a.get("kv_heads") or a["heads"]), int(a["dim"]), int(a["vdim"]),
+                                float(a["scale"]) if "scale" in a else int(a["dim"]) ** -0.5,
+                                float(a.get("softcap") or 0.0), rot, talk=True, bias=True)
+            right = DeltaSpec(int(r["heads"]), int(r.get("kv_heads") or r["heads"]), int(r["dim"]), int(r["vdim"]),
+                              int(r.get("conv") or 1))
+            for nm, sp in (("left", left), ("right", right)):
+                if sp.heads % sp.kv_heads:
+                    raise ValueError(f"Babotar layer {i} {nm}: {sp.heads} heads on {sp.kv_heads} key heads")
+            mixer = ParallelMixerSpec(left, right, float(m.get("left_scale", 1.0)), float(m.get("right_scale", 1.0)))
+        else:
+            raise ValueError(f"Babotar layer {i}: unsupported mixer type {typ!r}")
+        f, mlp = L.get("mlp"), None
+        if f is not None:
+            if f.get("kind", "dense") != "dense":
+                raise ValueError(f"Babotar layer {i}: unsupported feed-forward kind {f.get('kind')!r}")
+            mlp = DenseMLPSpec(int(f["ff"]))
+        specs.append(LayerSpec(mixer, mlp))
+    if not specs:
+        raise ValueError("Babotar: no layers")
+    heads = [s.mixer.left.heads if s.mixer.kind == "parallel" else s.mixer.heads for s in specs]
+    return cls(
+        model_type="babotar", vocab_size=int(d["vocab"]), hidden_size=int(d["width"]), num_layers=len(specs),
+        num_heads=max(heads), num_kv_heads=1, head_dim=1,
+        intermediate_size=max([s.mlp.ff for s in specs if s.mlp] or [0]),
+        max_position_embeddings=int(d["max_positions"]), norm="layernorm", norm_eps=float(d["norm"]["eps"]),
+        activation="gelu_tanh_glu", position="learned", rotary_dim=0, parallel_block=False,
+        tie_word_embeddings=False, layer_specs=specs, residual_fp32=True, streams=int(d.get("streams") or 0),
+        residual_mult=float(d.get("residual_mult", 1.0)), canon_taps=int((d.get("canon") or {}).get("taps") or 0),
+        bos_token_id=d.get("bos_token_id"), eos_token_id=_first(d.get("eos_token_id")),
+        pad_token_id=d.get("pad_token_id"),
+    )
+
+
 def _first(x):
     if isinstance(x, (list, tuple)):
         return x[0] if x else None
@@ -326,6 +463,22 @@ _PRESETS: Dict[str, Dict[str, Any]] = {
                                   mixer=dict(heads=3, dim=8, vdim=12, kv_rank=24, scale=0.3, mask=dict(size=5),
                                              kv_from=0),
                                   mlp=dict(kind="moe", router=dict(experts=4, top=1), expert=dict(ff=16, limit=2.0))),
+                         ]),
+    # sequential per-layer design: two residual streams, input convolution, a parallel (attention | delta rule) layer,
+    # a decay layer without a feed-forward, grouped heads and partial rotation
+    "tiny-babotar": dict(architecture="Babotar", vocab=211, width=48, max_positions=256, norm=dict(eps=1e-5),
+                         residual_mult=0.5, streams=2, canon=dict(taps=3),
+                         layers=[
+                             dict(type="parallel",
+                                  mixer=dict(left=dict(heads=4, kv_heads=2, dim=16, vdim=12, scale=0.2, softcap=30.0,
+                                                       rot=dict(base=1000.0, dims=8,
+                                                                scaling=dict(factor=4.0, original=64, fast=16.0,
+                                                                             slow=1.0))),
+                                             right=dict(heads=4, kv_heads=2, dim=8, vdim=12, conv=4),
+                                             left_scale=0.7, right_scale=1.1),
+                                  mlp=dict(kind="dense", ff=64)),
+                             dict(type="lightning", mixer=dict(heads=3, dim=8, vdim=16, decay=[0.5, 0.9, 0.99]),
+                                  mlp=None),
                          ]),
     # TP up to 8 (16 q / kv heads: 2 per rank at TP=8, as Llama-2-7B's 32 give 4)
     "tiny-llama16h": dict(model_type="llama", hidden_size=256, num_hidden_layers=2, num_attention_heads=16,

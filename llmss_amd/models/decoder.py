@@ -66,6 +66,7 @@ class StepInput:
     num_decode: int = 0  # extend: leading single-token decode rows
     has_prefix: bool = False  # extend: a prompt chunk continues a cached prefix
     cu_host: Optional[Sequence[int]] = None  # prefill: cu_seqlens on the host (micro-batch split points)
+    state_slots: Optional[torch.Tensor] = None  # [B] int32: per sequence (order of block_tables) its state slot, -1 none
 
 
 class StreamLedger:

@@ -1,14 +1,26 @@
 """Decoder whose layers are described one by one (``ModelConfig.layer_specs``) over an fp32 residual stream.
 
-The uniform families run through :class:`~llmss_amd.models.decoder.DecoderLM`; a per-layer design (Timisun) runs
-through :class:`LayeredLM`, which offers the engine the same surface (``hidden_states`` / ``logits`` over a
+The uniform families run through :class:`~llmss_amd.models.decoder.DecoderLM`; a per-layer design (Timisun, Babotar)
+runs through :class:`LayeredLM`, which offers the engine the same surface (``hidden_states`` / ``logits`` over a
 :class:`StepInput`, ``allocate_kv_cache``, ``kv_bytes_per_block``, ``plan``) and so shares its scheduler, paged
-cache pool, decode graphs and sampler. Each layer is a parallel block
+cache pool, decode graphs and sampler. A layer is either a parallel block (``cfg.parallel_block``)
 
     h = norm(x) ;  x <- x + (mixer(h) + ffn(h))          x fp32, norm weight stored around zero
 
-with the mixer and the feed-forward looked up by kind (``MIXERS`` / ``FFNS``), so another design can combine the
-same mechanisms with other constants or add its own beside them.
+or a sequential one over S residual streams x_1 .. x_S (S = 1: the ordinary pre-norm residual), per sublayer
+
+    u = sum_s in[s] x_s ;  y = sublayer(norm(u)) ;  x_t <- sum_s mix[s, t] x_s + c * out[t] * y
+
+where the mixer may read h + causal_conv(h) instead of h. The mixer and the feed-forward are looked up by kind
+(``MIXERS`` / ``FFNS``), so another design can combine the same mechanisms with other constants or add its own
+beside them. Besides pages of the shared pool a mixer may own per-sequence state (a matrix state per head, the last
+inputs of a convolution): ``LayerCache.state`` tensors indexed by the scheduler's state slot of each sequence
+(``StepInput.state_slots``); a portion that starts at position 0 starts from an empty state.
+
+Mixer ``parallel`` (ops: linear_f, rope_bias_cache, sink_attn, talk_mix, causal_conv, delta_recurrence,
+gated_group_norm): softmax attention with a sink, soft cap, partial scaled rotation and head mixing beside a gated
+delta rule, one input GEMM and one output GEMM for both. Mixer ``lightning`` (decay_recurrence, gated_group_norm):
+linear attention with a constant decay per head. Feed-forward ``dense`` (glu_act): gated, tanh-form GELU.
 
 Mixer ``latent_attention`` (ops: linear_f, latent_norm_cache, head_absorb, latent_attn, head_expand): the layer
 caches one RMS-normed latent row c per token in its paged cache ([blocks, block_size, kv_rank], the step's slots)
@@ -85,8 +97,97 @@ class MoEFeedForward:
                                combine=False)
 
 
-MIXERS = {"latent_attention": LatentAttention}
-FFNS = {"moe": MoEFeedForward}
+class ParallelMixer:
+    """Mixer ``parallel``: sink attention (paged k / v rows) beside a gated delta rule (matrix state and convolution
+    tail per sequence)."""
+
+    @staticmethod
+    def cache_row(spec) -> Optional[int]:
+        return spec.left.kv_heads * (spec.left.dim + spec.left.vdim)
+
+    @staticmethod
+    def allocate(model: "LayeredLM", spec, num_blocks: int, block_size: int, num_slots: int):
+        a, r = spec.left, spec.right
+        dt, dev = model.dtype, model.device
+        C = 2 * r.kv_heads * r.dim + r.heads * r.vdim
+        return (torch.zeros(num_blocks, block_size, a.kv_heads * a.dim, dtype=dt, device=dev),
+                torch.zeros(num_blocks, block_size, a.kv_heads * a.vdim, dtype=dt, device=dev),
+                {"S": torch.zeros(num_slots, r.heads, r.dim, r.vdim, dtype=torch.float32, device=dev),
+                 "tail": torch.zeros(num_slots, max(r.conv - 1, 0), C, dtype=torch.float32, device=dev)})
+
+    @staticmethod
+    def state_bytes(spec) -> int:
+        r = spec.right
+        return 4 * (r.heads * r.dim * r.vdim + max(r.conv - 1, 0) * (2 * r.kv_heads * r.dim + r.heads * r.vdim))
+
+    @staticmethod
+    def forward(model: "LayeredLM", i: int, W, spec, h, inp: StepInput, cu, caches):
+        dt, eps = model.dtype, model.cfg.norm_eps
+        a, r, c = spec.left, spec.right, W.cols
+        kc, vc, st = caches[i]
+        T = h.shape[0]
+        proj = ops.linear_f(h, W.proj, dt)
+        # left: softmax attention with a sink over the paged cache, the heads' weights mixed afterwards
+        q = ops.rope_bias_cache(proj, c["lq"], c["lk"], c["lv"], W.bias, inp.positions, W.angles,
+                                a.rot.dims if a.rot is not None else 0, kc, vc, inp.slots, a.heads, a.kv_heads, a.dim,
+                                a.vdim)
+        O = ops.sink_attn(q, kc, vc, inp.block_tables, cu, inp.ctx_lens, a.heads, a.kv_heads, a.dim, a.vdim, a.scale,
+                          a.softcap, W.talk is not None)
+        nl, nr = a.heads * a.vdim, r.heads * r.vdim
+        both = torch.empty(T, nl + nr, dtype=dt, device=h.device)  # [left | right] rows for the one output GEMM
+        ops.talk_mix(O, W.talk, spec.left_scale, a.heads, a.kv_heads, a.vdim, out=both[:, :nl])
+        # right: short convolution + SiLU on q | k | v, then the gated delta rule over the sequence's matrix state
+        nqk = r.kv_heads * r.dim
+        qkv = ops.causal_conv(proj[:, c["rq"]:c["rq"] + 2 * nqk + nr], W.conv, st["tail"], cu, inp.ctx_lens,
+                              inp.state_slots, False, True, torch.float32)
+        o = ops.delta_recurrence(qkv[:, :nqk], qkv[:, nqk:2 * nqk], qkv[:, 2 * nqk:], proj[:, c["ra"]:c["ra"] + r.heads],
+                                 proj[:, c["rb"]:c["rb"] + r.heads], W.A_log, W.dt_bias, st["S"], cu, inp.ctx_lens,
+                                 inp.state_slots, r.heads, r.kv_heads, r.dim, r.vdim)
+        ops.gated_group_norm(o, proj[:, c["rg"]:c["rg"] + nr], W.norm, eps, "silu", spec.right_scale,
+                             out=both[:, nl:])
+        return ops.linear_f(both, W.o, dt)
+
+
+class DecayMixer:
+    """Mixer ``lightning``: S <- decay_h S + k v^T, o = S^T q per head, then a gated RMS norm over all heads."""
+
+    @staticmethod
+    def cache_row(spec) -> Optional[int]:
+        return None
+
+    @staticmethod
+    def allocate(model: "LayeredLM", spec, num_blocks: int, block_size: int, num_slots: int):
+        return (None, None, {"S": torch.zeros(num_slots, spec.heads, spec.dim, spec.vdim, dtype=torch.float32,
+                                              device=model.device)})
+
+    @staticmethod
+    def state_bytes(spec) -> int:
+        return 4 * spec.heads * spec.dim * spec.vdim
+
+    @staticmethod
+    def forward(model: "LayeredLM", i: int, W, spec, h, inp: StepInput, cu, caches):
+        dt, c = model.dtype, W.cols
+        nqk, nv = spec.heads * spec.dim, spec.heads * spec.vdim
+        proj = ops.linear_f(h, W.proj, dt)
+        o = ops.decay_recurrence(proj[:, c["q"]:c["q"] + nqk], proj[:, c["k"]:c["k"] + nqk],
+                                 proj[:, c["v"]:c["v"] + nv], W.decay, caches[i][2]["S"], cu, inp.ctx_lens,
+                                 inp.state_slots, spec.heads, spec.dim, spec.vdim, True)
+        y = ops.gated_group_norm(o, proj[:, c["g"]:c["g"] + nv], W.norm, model.cfg.norm_eps, "sigmoid", 1.0,
+                                 out_dtype=dt)
+        return ops.linear_f(y, W.o, dt)
+
+
+class DenseFeedForward:
+    """Feed-forward ``dense``: down(act(gate h) * (up h)), gate and up as one GEMM."""
+
+    @staticmethod
+    def forward(model: "LayeredLM", W, spec, h):
+        dt = model.dtype
+        return ops.linear_f(ops.glu_act(ops.linear_f(h, W.gu, dt), spec.ff, spec.act), W.down, dt)
+
+
+MIXERS = {"latent_attention": LatentAttention, "parallel": ParallelMixer, "lightning": DecayMixer}
+FFNS = {"moe": MoEFeedForward, "dense": DenseFeedForward}
 
 
 class LayeredLM:
@@ -143,11 +244,12 @@ class LayeredLM:
             if K % 16 == 0 and N % 8 == 0 and (N, K) not in {(s.N, s.K) for s in out.values()}:
                 out[f"{name}_{N}x{K}"] = GemmShape(N, K)
         for L in self.w.layers:
-            put("qc", L.mix.qc)
-            put("o", L.mix.o)
-            if L.mlp is not None and L.mlp.shared_gu is not None:
-                put("shared_gu", L.mlp.shared_gu)
-                put("shared_down", L.mlp.shared_down)
+            for nm in ("qc", "proj", "o"):
+                if hasattr(L.mix, nm):
+                    put(nm, getattr(L.mix, nm))
+            for nm in ("shared_gu", "shared_down", "gu", "down"):
+                if L.mlp is not None and getattr(L.mlp, nm, None) is not None and getattr(L.mlp, nm).dim() == 2:
+                    put(nm, getattr(L.mlp, nm))
         put("head", self.w.head.w)
         return out
 
@@ -156,16 +258,38 @@ class LayeredLM:
         return [MIXERS[s.mixer.kind].cache_row(s.mixer) for s in self.cfg.layer_specs]
 
     def kv_bytes_per_block(self, block_size: int) -> int:
-        return sum(block_size * r * self.w.wte.element_size() for r in self._cache_rows() if r)
+        return max(1, sum(block_size * r * self.w.wte.element_size() for r in self._cache_rows() if r))
 
-    def allocate_kv_cache(self, num_blocks: int, block_size: int):
-        """One (rows, None) pair per layer; a layer that reads another layer's rows holds that layer's pair."""
+    @property
+    def needs_state(self) -> bool:
+        """Some mixer keeps per-sequence state besides its pages: steps must carry the sequences' state slots."""
+        return any(hasattr(MIXERS[s.mixer.kind], "state_bytes") for s in self.cfg.layer_specs) or \
+            bool(self.cfg.canon_taps > 1)
+
+    def state_bytes_per_slot(self) -> int:
+        n = sum(MIXERS[s.mixer.kind].state_bytes(s.mixer) for s in self.cfg.layer_specs
+                if hasattr(MIXERS[s.mixer.kind], "state_bytes"))
+        return n + 4 * max(self.cfg.canon_taps - 1, 0) * self.cfg.hidden_size * len(self.cfg.layer_specs)
+
+    def allocate_kv_cache(self, num_blocks: int, block_size: int, num_slots: int = 0):
+        """One entry per layer. Latent attention: (rows, None), a layer that reads another layer's rows holding that
+        layer's pair. Mixers with an ``allocate`` of their own: (key pages, value pages, {name: per-slot state});
+        ``num_slots`` state slots, one per running sequence. The input convolution's tails of all layers live in
+        ``self.canon_tail`` [layers, slots, taps - 1, W]."""
         caches: list = []
         for s, r in zip(self.cfg.layer_specs, self._cache_rows()):
-            if r:
+            mx = MIXERS[s.mixer.kind]
+            if hasattr(mx, "allocate"):
+                if num_slots <= 0:
+                    raise ValueError(f"{self.cfg.model_type}: the cache needs state slots (num_slots)")
+                caches.append(mx.allocate(self, s.mixer, num_blocks, block_size, num_slots))
+            elif r:
                 caches.append((torch.zeros(num_blocks, block_size, r, dtype=self.dtype, device=self.device), None))
             else:
                 caches.append(caches[s.mixer.kv_from])
+        if self.cfg.canon_taps > 1:
+            self.canon_tail = torch.zeros(len(caches), max(num_slots, 1), self.cfg.canon_taps - 1,
+                                          self.cfg.hidden_size, dtype=torch.float32, device=self.device)
         return caches
 
     # ---------------------------------------------------------------------------- forward
@@ -186,9 +310,11 @@ class LayeredLM:
         return inp.cu_seqlens
 
     def hidden_states(self, inp: StepInput, kv_caches) -> torch.Tensor:
-        if inp.block_tables is None or inp.ctx_lens is None or kv_caches[0][0] is None:
+        if inp.block_tables is None or inp.ctx_lens is None or not any(t is not None for t in kv_caches[0]):
             raise ValueError(f"{self.cfg.model_type} attends through its paged cache: the step needs block tables, "
                              f"context lengths and a cache (a cache-less recompute step is not supported)")
+        if not self.cfg.parallel_block:
+            return self._sequential_blocks(inp, kv_caches)
         cfg, w = self.cfg, self.w
         eps, off, dt = cfg.norm_eps, cfg.norm_offset, self.dtype
         cu = self._cu(inp)
@@ -203,6 +329,34 @@ class LayeredLM:
         h = ops.resid_add_norm(x, a, f, w.lnf_w, off, eps, dt)
         if self.tap is not None:
             self.tap(len(w.layers) - 1, x)
+        return h
+
+    def _sequential_blocks(self, inp: StepInput, kv_caches) -> torch.Tensor:
+        """Sequential blocks over the residual streams. The write-back of one sublayer and the read + norm of the
+        next are one op (stream_add_norm), as the residual add and the next norm are for the other families."""
+        cfg, w, dt = self.cfg, self.w, self.dtype
+        if self.needs_state and inp.state_slots is None:
+            raise ValueError(f"{cfg.model_type} keeps per-sequence state: the step needs the sequences' state slots")
+        eps, c, rms = cfg.norm_eps, cfg.residual_mult, cfg.norm == "rmsnorm"
+        cu = self._cu(inp)
+        x = ops.embed_streams(inp.input_ids, inp.positions, w.wte, w.wpe, max(cfg.streams, 1))
+        y = prev = None  # the sublayer output not yet written back, and its stream weights
+        for i, (L, spec) in enumerate(zip(w.layers, cfg.layer_specs)):
+            canon = L.canon is not None
+            h = ops.stream_add_norm(x, y, prev.mix if prev else None, prev.outw if prev else None, c, L.hc1.inw,
+                                    L.norm1, eps, rms, torch.float32 if canon else dt)
+            if self.tap is not None and i:
+                self.tap(i - 1, x.sum(0))
+            if canon:
+                tail = self.canon_tail[i] if cfg.canon_taps > 1 else None
+                h = ops.causal_conv(h, L.canon, tail, cu, inp.ctx_lens, inp.state_slots, True, False, dt)
+            y, prev = MIXERS[spec.mixer.kind].forward(self, i, L.mix, spec.mixer, h, inp, cu, kv_caches), L.hc1
+            if spec.mlp is not None:
+                h = ops.stream_add_norm(x, y, prev.mix, prev.outw, c, L.hc2.inw, L.norm2, eps, rms, dt)
+                y, prev = FFNS[spec.mlp.kind].forward(self, L.mlp, spec.mlp, h), L.hc2
+        h = ops.stream_add_norm(x, y, prev.mix, prev.outw, c, None, w.lnf_w, eps, rms, dt)
+        if self.tap is not None:
+            self.tap(len(w.layers) - 1, x.sum(0))
         return h
 
     @property

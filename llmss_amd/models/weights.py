@@ -711,3 +711,258 @@ def _timisun_random(cfg: ModelConfig, seed: int, device="cpu"):
         t = 1.0 + 0.1 * t if std is None else t * std
         return t.to(torch.bfloat16).float()
     return get
+
+
+# ------------------------------------------------------------------------------ sequential per-layer designs (Babotar)
+@dataclass
+class StreamWeights:
+    """Read / write / mix weights of one sublayer over the residual streams (fp32): u = sum_s inw[s] x_s;
+    x_t <- sum_s mix[s, t] x_s + c * outw[t] * y."""
+    inw: torch.Tensor
+    outw: torch.Tensor
+    mix: torch.Tensor
+
+    def tensors(self):
+        return [self.inw, self.outw, self.mix]
+
+
+@dataclass
+class ParallelMixWeights:
+    """Attention beside a gated delta rule, both reading the same rows. ``proj`` [N padded to 8, W] holds every input
+    projection of the two as one matrix (one GEMM); ``cols`` names the first column of each part: lq, lk, lv (the
+    attention's q, k, v, contiguous), rq, rk, rv (the delta rule's, contiguous: one convolution runs over them), rg
+    (its output gate), rb, ra (its per-head write strength and decay inputs). ``bias`` [lq | lk | lv] or None;
+    ``talk`` fp32 [heads, heads] or None; ``angles`` fp32 [positions, rot / 2, 2] or None; ``conv`` [rq | rk | rv
+    channels, taps]; ``A_log``, ``dt_bias`` fp32 [heads]; ``norm`` [vdim]; ``o`` [W, left width + right width], the
+    two output projections side by side (one GEMM over the concatenated branch outputs)."""
+    proj: torch.Tensor
+    cols: Dict[str, int]
+    bias: Optional[torch.Tensor]
+    talk: Optional[torch.Tensor]
+    angles: Optional[torch.Tensor]
+    conv: torch.Tensor
+    A_log: torch.Tensor
+    dt_bias: torch.Tensor
+    norm: torch.Tensor
+    o: torch.Tensor
+
+    def tensors(self):
+        return [t for t in (self.proj, self.bias, self.talk, self.angles, self.conv, self.A_log, self.dt_bias, self.norm,
+                            self.o) if t is not None]
+
+
+@dataclass
+class DecayMixWeights:
+    """Decay linear attention: ``proj`` [q | k | v | g rows padded to 8, W], ``decay`` fp32 [heads], ``norm``
+    [heads * vdim], ``o`` [W, heads * vdim]."""
+    proj: torch.Tensor
+    cols: Dict[str, int]
+    decay: torch.Tensor
+    norm: torch.Tensor
+    o: torch.Tensor
+
+    def tensors(self):
+        return [self.proj, self.decay, self.norm, self.o]
+
+
+@dataclass
+class DenseMLPWeights:
+    """``gu`` [2 ff, W]: gate rows, then up rows; ``down`` [W, ff]."""
+    gu: torch.Tensor
+    down: torch.Tensor
+
+    def tensors(self):
+        return [self.gu, self.down]
+
+
+@dataclass
+class SeqBlockWeights:
+    """One sequential block: norm1 -> (input convolution) -> mixer, norm2 -> feed-forward, each over the streams."""
+    norm1: torch.Tensor
+    norm2: Optional[torch.Tensor]
+    hc1: StreamWeights
+    hc2: Optional[StreamWeights]
+    canon: Optional[torch.Tensor]
+    mix: object
+    mlp: Optional[DenseMLPWeights]
+
+    def tensors(self):
+        out = [self.norm1] + self.hc1.tensors() + self.mix.tensors()
+        for t in (self.norm2, self.canon):
+            if t is not None:
+                out.append(t)
+        if self.hc2 is not None:
+            out += self.hc2.tensors()
+        if self.mlp is not None:
+            out += self.mlp.tensors()
+        return out
+
+
+def babotar_shapes(cfg: ModelConfig) -> Dict[str, tuple]:
+    """Checkpoint tensor names of a Babotar config and their shapes."""
+    W, S = cfg.hidden_size, cfg.streams
+    out = {"embed": (cfg.vocab_size, W), "pos": (cfg.max_position_embeddings, W), "final.norm": (W,),
+           "head": (cfg.vocab_size, W)}
+    for i, spec in enumerate(cfg.layer_specs):
+        p = f"l{i}."
+        out[p + "norm1"] = (W,)
+        subs = (1, 2) if spec.mlp is not None else (1,)
+        if S:
+            for q in subs:
+                out.update({f"{p}hc{q}.in": (S,), f"{p}hc{q}.out": (S,), f"{p}hc{q}.mix": (S, S)})
+        if cfg.canon_taps:
+            out[p + "canon1"] = (W, cfg.canon_taps)
+        m = spec.mixer
+        if m.kind == "lightning":
+            out.update({p + "mix.q": (m.heads * m.dim, W), p + "mix.k": (m.heads * m.dim, W),
+                        p + "mix.v": (m.heads * m.vdim, W), p + "mix.g": (m.heads * m.vdim, W),
+                        p + "mix.o": (W, m.heads * m.vdim), p + "mix.norm": (m.heads * m.vdim,)})
+        else:
+            a, r, pl, pr = m.left, m.right, p + "mix.left.", p + "mix.right."
+            out.update({pl + "q": (a.heads * a.dim, W), pl + "k": (a.kv_heads * a.dim, W),
+                        pl + "v": (a.kv_heads * a.vdim, W), pl + "o": (W, a.heads * a.vdim)})
+            if a.bias:
+                out.update({pl + "q.b": (a.heads * a.dim,), pl + "k.b": (a.kv_heads * a.dim,),
+                            pl + "v.b": (a.kv_heads * a.vdim,)})
+            if a.talk:
+                out[pl + "talk"] = (a.heads, a.heads)
+            out.update({pr + "q": (r.kv_heads * r.dim, W), pr + "q.conv": (r.kv_heads * r.dim, r.conv),
+                        pr + "k": (r.kv_heads * r.dim, W), pr + "k.conv": (r.kv_heads * r.dim, r.conv),
+                        pr + "v": (r.heads * r.vdim, W), pr + "v.conv": (r.heads * r.vdim, r.conv),
+                        pr + "b": (r.heads, W), pr + "a": (r.heads, W), pr + "A_log": (r.heads,),
+                        pr + "dt_bias": (r.heads,), pr + "norm": (r.vdim,), pr + "g": (r.heads * r.vdim, W),
+                        pr + "o": (W, r.heads * r.vdim)})
+        if spec.mlp is not None:
+            out.update({p + "norm2": (W,), p + "mlp.gate": (spec.mlp.ff, W), p + "mlp.up": (spec.mlp.ff, W),
+                        p + "mlp.down": (W, spec.mlp.ff)})
+    return out
+
+
+def _cat_rows(parts, pad_to: int = 8):
+    """(matrix of the parts' rows one after the other, zero rows up to a multiple of ``pad_to``; first row of each)."""
+    cols, n = {}, 0
+    for name, t in parts:
+        cols[name] = n
+        n += t.shape[0]
+    mats = [t for _, t in parts]
+    if n % pad_to:
+        mats.append(torch.zeros(pad_to - n % pad_to, mats[0].shape[1], dtype=mats[0].dtype))
+    return torch.cat(mats, 0), cols
+
+
+def _babotar_finish(cfg: ModelConfig, get, has, device, dtype) -> ModelWeights:
+    """``get(name)`` returns the checkpoint tensor of that name (CPU), ``has(name)`` whether it exists. Shapes are
+    checked against the config; the head-mixing matrix and the q / k / v biases are optional tensors."""
+    from ..ops.reference import rope_angle_table
+
+    shapes = babotar_shapes(cfg)
+    optional = (".talk", ".q.b", ".k.b", ".v.b")
+
+    def g(name):
+        t = get(name)
+        if tuple(t.shape) != shapes[name]:
+            raise ValueError(f"{name} has shape {tuple(t.shape)}, the config says {shapes[name]}")
+        return t
+
+    def opt(name):
+        return g(name) if has(name) else None
+
+    def dev(t, dt=dtype):
+        return None if t is None else t.to(device=device, dtype=dt).contiguous()
+
+    def f32(t):
+        return dev(t, torch.float32)
+    W, S = cfg.hidden_size, cfg.streams
+    one = StreamWeights(f32(torch.ones(1)), f32(torch.ones(1)), f32(torch.ones(1, 1)))
+    tables = {}
+    layers = []
+    for i, spec in enumerate(cfg.layer_specs):
+        p = f"l{i}."
+
+        def hc(q):
+            return StreamWeights(f32(g(f"{p}hc{q}.in")), f32(g(f"{p}hc{q}.out")), f32(g(f"{p}hc{q}.mix"))) if S else one
+        m = spec.mixer
+        if m.kind == "lightning":
+            proj, cols = _cat_rows([(n, g(p + "mix." + n)) for n in ("q", "k", "v", "g")])
+            mix = DecayMixWeights(dev(proj), cols, f32(torch.tensor(m.decay)), dev(g(p + "mix.norm")),
+                                  dev(g(p + "mix.o")))
+        else:
+            a, pl, pr = m.left, p + "mix.left.", p + "mix.right."
+            proj, cols = _cat_rows([("lq", g(pl + "q")), ("lk", g(pl + "k")), ("lv", g(pl + "v")),
+                                    ("rq", g(pr + "q")), ("rk", g(pr + "k")), ("rv", g(pr + "v")),
+                                    ("rg", g(pr + "g")), ("rb", g(pr + "b")), ("ra", g(pr + "a"))])
+            bias = None
+            if any(has(pl + n + ".b") for n in "qkv"):
+                bias = torch.cat([g(pl + n + ".b") if has(pl + n + ".b") else torch.zeros(shapes[pl + n][0])
+                                  for n in "qkv"])
+            angles = None
+            if a.rot is not None and a.rot.dims:
+                key = (a.rot.dims, a.rot.base, a.rot.scaling)
+                if key not in tables:
+                    tables[key] = dev(rope_angle_table(cfg.max_position_embeddings, *key), torch.float32)
+                angles = tables[key]
+            mix = ParallelMixWeights(
+                dev(proj), cols, dev(bias), f32(opt(pl + "talk")), angles,
+                dev(torch.cat([g(pr + n + ".conv") for n in "qkv"], 0)), f32(g(pr + "A_log")), f32(g(pr + "dt_bias")),
+                dev(g(pr + "norm")), dev(torch.cat([g(pl + "o"), g(pr + "o")], 1)))
+        mlp = None
+        if spec.mlp is not None:
+            mlp = DenseMLPWeights(dev(torch.cat([g(p + "mlp.gate"), g(p + "mlp.up")], 0)), dev(g(p + "mlp.down")))
+        layers.append(SeqBlockWeights(
+            dev(g(p + "norm1")), dev(g(p + "norm2")) if mlp is not None else None, hc(1),
+            hc(2) if mlp is not None else None, dev(g(p + "canon1")) if cfg.canon_taps else None, mix, mlp))
+    vp = math.ceil(cfg.vocab_size / 16) * 16
+    head = torch.zeros(vp, W, dtype=dtype, device=device)
+    head[:cfg.vocab_size].copy_(g("head").to(device=device, dtype=dtype))
+    return ModelWeights(wte=dev(g("embed")), wpe=dev(g("pos")) if has("pos") else None, layers=layers,
+                        lnf_w=dev(g("final.norm")), lnf_b=None, head=Linear(head))
+
+
+def load_babotar_weights(cfg: ModelConfig, reader, device="cpu", dtype=torch.bfloat16) -> ModelWeights:
+    names = set(reader.keys())
+    return _babotar_finish(cfg, lambda n: reader.get(n), lambda n: n in names, device, dtype)
+
+
+def _babotar_random(cfg: ModelConfig, seed: int, device="cpu"):
+    import zlib
+
+    shapes = babotar_shapes(cfg)
+
+    def get(name: str) -> torch.Tensor:
+        g = torch.Generator(device=device)
+        g.manual_seed((seed * 1000003 + zlib.crc32(name.encode())) & 0x7FFFFFFF)
+        shp = shapes[name]
+        t = torch.randn(*shp, generator=g, dtype=torch.float32, device=device)
+        last = name.split(".")[-1]
+        if last.startswith("norm") or name == "final.norm":
+            t = 1.0 + 0.1 * t
+        elif name == "pos":
+            t = 0.3 * t
+        elif last in ("in", "out"):
+            t = 1.0 / max(1, cfg.streams) + 0.2 * t if last == "in" else 1.0 + 0.2 * t
+        elif last == "mix":
+            t = torch.eye(shp[0], device=device) + 0.15 * t
+        elif last == "talk":
+            t = torch.eye(shp[0], device=device) + 0.2 * t
+        elif last in ("conv", "canon1"):
+            t = t * shp[1] ** -0.5
+        elif last == "A_log":
+            t = 0.5 * t - 1.0
+        elif last in ("dt_bias", "b") and len(shp) == 1:
+            t = 0.3 * t
+        elif len(shp) == 2 and name not in ("embed",):
+            t = t * shp[1] ** -0.5
+        return t.to(torch.bfloat16).float()
+    return get
+
+
+def random_babotar_weights(cfg: ModelConfig, device="cpu", dtype=torch.bfloat16, seed: int = 0) -> ModelWeights:
+    """Random-init weights of a Babotar config (values rounded to bf16, so a bf16 and an fp32 run hold the same
+    model): projections ~ N(0, 1 / fan_in), norm weights around one, stream weights around the plain residual."""
+    return _babotar_finish(cfg, _babotar_random(cfg, seed), lambda n: True, device, dtype)
+
+
+def babotar_state_dict(cfg: ModelConfig, seed: int = 0) -> Dict[str, torch.Tensor]:
+    """The random weights of :func:`random_babotar_weights` under their checkpoint names (bf16; tests, examples)."""
+    get = _babotar_random(cfg, seed)
+    return {n: get(n).to(torch.bfloat16) for n in babotar_shapes(cfg)}

@@ -174,3 +174,16 @@ glu_clamp = _route("glu_clamp")
 moe_route = _route("moe_route")
 moe_router = _route("moe_router")
 moe_experts = _route("moe_experts")
+
+# ------------------------------- residual streams / convolution tails / matrix-state recurrences / sink attention
+embed_streams = _route("embed_streams")
+stream_add_norm = _route("stream_add_norm")
+causal_conv = _route("causal_conv")
+gated_group_norm = _route("gated_group_norm")
+glu_act = _route("glu_act")
+decay_recurrence = _route("decay_recurrence")
+delta_recurrence = _route("delta_recurrence")
+rope_bias_cache = _route("rope_bias_cache")
+sink_attn = _route("sink_attn")
+talk_mix = _route("talk_mix")
+rope_angle_table = ref.rope_angle_table

@@ -1074,3 +1074,220 @@ def moe_experts(h, idx, wts, gate, up, down, limit, alpha, shared=None, combine=
     L.moe_combine(y.data_ptr(), place.data_ptr(), wts.data_ptr(), _ptr(shared),
                   shared.stride(0) if shared is not None else 0, out.data_ptr(), T, N, top, dt, st)
     return out
+
+
+# ----------------------------------- residual streams / convolution tails / matrix-state recurrences / sink attention
+def _i32(t, name, n=None):
+    _check(t.dtype == torch.int32 and t.is_contiguous() and t.is_cuda, f"{name} must be contiguous int32 cuda")
+    if n is not None:
+        _check(t.numel() >= n, f"{name} too short")
+
+
+def _f32c(t, name):
+    _check(t.dtype == torch.float32 and t.is_contiguous() and t.is_cuda, f"{name} must be contiguous fp32 cuda")
+
+
+def embed_streams(ids, positions, table, pos_table, streams):
+    T = ids.numel()
+    V, W = table.shape
+    for t, nm in ((ids, "ids"), (positions, "positions")):
+        _check(t.dtype == torch.int64 and t.is_contiguous() and t.is_cuda and t.numel() == T, f"{nm}: int64 [T] cuda")
+    _check(table.is_contiguous(), "embedding table contiguous")
+    if pos_table is not None:
+        _check(pos_table.is_contiguous() and pos_table.dtype == table.dtype and pos_table.shape[1] == W,
+               "position table [positions, W] in the table's storage type")
+    x = torch.empty(streams, T, W, dtype=torch.float32, device=table.device)
+    lib().embed_streams(ids.data_ptr(), positions.data_ptr(), table.data_ptr(), _ptr(pos_table), x.data_ptr(),
+                        int(streams), T, W, V, pos_table.shape[0] if pos_table is not None else 1, _dt(table, "table"),
+                        _stream())
+    return x
+
+
+def stream_add_norm(x, y, mix, outw, c, inw, w, eps, rms, out_dtype):
+    S, T, W = x.shape
+    _check(x.dtype == torch.float32 and x.is_contiguous() and x.is_cuda, "x fp32 [S, T, W] contiguous")
+    dt = None
+    if y is not None:
+        _rows(y, "y", W)
+        _check(y.shape[0] == T, "y rows")
+        _f32c(mix, "mix")
+        _f32c(outw, "outw")
+        _check(mix.numel() == S * S and outw.numel() == S, "mix [S, S], outw [S]")
+        dt = y.dtype
+    h = None
+    if w is not None:
+        _check(w.is_contiguous() and w.numel() == W and w.is_cuda, "norm weight [W]")
+        _check(dt is None or w.dtype == dt, "norm weight in y's storage type")
+        dt = w.dtype
+        if inw is not None:
+            _f32c(inw, "inw")
+            _check(inw.numel() == S, "inw [S]")
+        _check(out_dtype in (dt, torch.float32), "h in the storage type or fp32")
+        h = torch.empty(T, W, dtype=out_dtype, device=x.device)
+    if dt is None or T == 0:
+        return h
+    _check(dt in _DT, "storage type bf16 / fp32")
+    lib().stream_add_norm(x.data_ptr(), _ptr(y), y.stride(0) if y is not None else 0, _ptr(mix), _ptr(outw), float(c),
+                          _ptr(inw) if w is not None else 0, _ptr(w), float(eps), int(bool(rms)), _ptr(h), W, S, T, W,
+                          _DT[dt], int(h is not None and h.dtype == torch.float32), _stream())
+    return h
+
+
+def causal_conv(x, w, state, cu, ctx_lens, state_slots, residual, silu, out_dtype):
+    T, C = x.shape
+    _rows(x, "x")
+    taps = w.shape[1]
+    _check(w.shape[0] == C and w.is_contiguous() and w.is_cuda, "conv weight [C, taps]")
+    B = cu.numel() - 1
+    _i32(cu, "cu")
+    _i32(ctx_lens, "ctx_lens", B)
+    _i32(state_slots, "state_slots", B)
+    if taps > 1:
+        _f32c(state, "state")
+        _check(state.dim() == 3 and tuple(state.shape[1:]) == (taps - 1, C), "state [slots, taps - 1, C]")
+    out = torch.empty(T, C, dtype=out_dtype, device=x.device)
+    lib().causal_conv(x.data_ptr(), x.stride(0), w.data_ptr(), _ptr(state) if taps > 1 else 0, cu.data_ptr(),
+                      ctx_lens.data_ptr(), state_slots.data_ptr(), out.data_ptr(), C, T, B, C, taps,
+                      int(bool(residual)), int(bool(silu)), _dt(x, "x"), _dt(w, "w"), _DT[out_dtype], _stream())
+    return out
+
+
+def gated_group_norm(o, gate, w, eps, act, c, out=None, out_dtype=None):
+    T, N = o.shape
+    _rows(o, "o", dtype=torch.float32)
+    n = w.numel()
+    _check(N % n == 0 and w.is_contiguous(), "the group size (len(w)) must divide the row")
+    _rows(gate, "gate", N)
+    if out is None:
+        out = torch.empty(T, N, dtype=out_dtype, device=o.device)
+    _rows(out, "out", N)
+    _check(gate.dtype == w.dtype == out.dtype and gate.shape[0] == T and out.shape[0] == T, "gate / w / out types, rows")
+    lib().gated_group_norm(o.data_ptr(), o.stride(0), gate.data_ptr(), gate.stride(0), w.data_ptr(), float(eps),
+                           {"sigmoid": 0, "silu": 1}[act], float(c), out.data_ptr(), out.stride(0), T, N // n, n,
+                           _dt(w, "w"), _stream())
+    return out
+
+
+def glu_act(gu, F, act):
+    T = gu.shape[0]
+    _rows(gu, "gu")
+    _check(gu.shape[1] >= 2 * F, "gate | up too narrow")
+    out = torch.empty(T, F, dtype=gu.dtype, device=gu.device)
+    lib().glu_act(gu.data_ptr(), gu.stride(0), out.data_ptr(), F, T, F, {"gelu_tanh": 0, "silu": 1}[act],
+                  _dt(gu, "gu"), _stream())
+    return out
+
+
+def _rec_common(q, k, v, state, cu, ctx_lens, state_slots, heads, kv_heads, dim, vdim):
+    T = q.shape[0]
+    for t, nm, cols in ((q, "q", kv_heads * dim), (k, "k", kv_heads * dim), (v, "v", heads * vdim)):
+        _rows(t, nm, cols)
+        _check(t.shape[0] == T and t.dtype == q.dtype, f"{nm} rows / type")
+    B = cu.numel() - 1
+    _i32(cu, "cu")
+    _i32(ctx_lens, "ctx_lens", B)
+    _i32(state_slots, "state_slots", B)
+    _f32c(state, "state")
+    _check(state.dim() == 4 and tuple(state.shape[1:]) == (heads, dim, vdim), "state [slots, heads, dim, vdim]")
+    return T, B, torch.empty(T, heads * vdim, dtype=torch.float32, device=q.device)
+
+
+def decay_recurrence(q, k, v, decay, state, cu, ctx_lens, state_slots, heads, dim, vdim, silu_in=True):
+    T, B, out = _rec_common(q, k, v, state, cu, ctx_lens, state_slots, heads, heads, dim, vdim)
+    _f32c(decay, "decay")
+    _check(decay.numel() == heads, "decay [heads]")
+    if T:
+        lib().recurrence(0, q.data_ptr(), k.data_ptr(), v.data_ptr(), q.stride(0), k.stride(0), v.stride(0), 0, 0, 0, 0,
+                         decay.data_ptr(), 0, state.data_ptr(), cu.data_ptr(), ctx_lens.data_ptr(),
+                         state_slots.data_ptr(), out.data_ptr(), heads * vdim, B, heads, heads, dim, vdim,
+                         int(bool(silu_in)), _dt(q, "q"), 0, _stream())
+    return out
+
+
+def delta_recurrence(q, k, v, a, b_, A_log, dt_bias, state, cu, ctx_lens, state_slots, heads, kv_heads, dim, vdim):
+    T, B, out = _rec_common(q, k, v, state, cu, ctx_lens, state_slots, heads, kv_heads, dim, vdim)
+    _f32c(A_log, "A_log")
+    _f32c(dt_bias, "dt_bias")
+    _check(A_log.numel() == heads and dt_bias.numel() == heads, "A_log, dt_bias [heads]")
+    _rows(a, "a", heads)
+    _rows(b_, "b", heads)
+    # a and b are columns of one projection: addressed from a's base with b's offset in elements
+    _check(a.dtype == b_.dtype and a.stride(0) == b_.stride(0) and a.shape[0] == T and b_.shape[0] == T
+           and a.untyped_storage().data_ptr() == b_.untyped_storage().data_ptr(), "a and b: columns of one tensor")
+    off_b = (b_.data_ptr() - a.data_ptr()) // a.element_size()
+    if T:
+        lib().recurrence(1, q.data_ptr(), k.data_ptr(), v.data_ptr(), q.stride(0), k.stride(0), v.stride(0),
+                         a.data_ptr(), a.stride(0), 0, int(off_b), A_log.data_ptr(), dt_bias.data_ptr(),
+                         state.data_ptr(), cu.data_ptr(), ctx_lens.data_ptr(), state_slots.data_ptr(), out.data_ptr(),
+                         heads * vdim, B, heads, kv_heads, dim, vdim, 0, _dt(q, "q"), _dt(a, "a"), _stream())
+    return out
+
+
+def rope_angle_table(npos, dims, base, scaling=None):
+    from . import reference as ref
+
+    return ref.rope_angle_table(npos, dims, base, scaling)
+
+
+def rope_bias_cache(proj, off_q, off_k, off_v, bias, positions, table, rot, k_cache, v_cache, slots, heads, kv_heads,
+                    dim, vdim):
+    T = proj.shape[0]
+    _rows(proj, "proj")
+    nq, nk, nv = heads * dim, kv_heads * dim, kv_heads * vdim
+    _check(min(off_q, off_k, off_v) >= 0 and max(off_q + nq, off_k + nk, off_v + nv) <= proj.shape[1],
+           "q / k / v columns outside the projection")
+    if bias is not None:
+        _check(bias.dtype == proj.dtype and bias.is_contiguous() and bias.numel() == nq + nk + nv, "bias q | k | v")
+    for c, n, nm in ((k_cache, nk, "k cache"), (v_cache, nv, "v cache")):
+        _check(c.dtype == proj.dtype and c.is_contiguous() and c.dim() == 3 and c.shape[2] == n,
+               f"{nm} [blocks, block_size, {n}] in the model's storage type")
+    for t, nm in ((positions, "positions"), (slots, "slots")):
+        _check(t.dtype == torch.int64 and t.is_contiguous() and t.is_cuda and t.numel() == T, f"{nm}: int64 [T] cuda")
+    npos = 1
+    if rot:
+        _f32c(table, "angle table")
+        _check(table.dim() == 3 and table.shape[1] == rot // 2 and table.shape[2] == 2, "angle table [npos, rot / 2, 2]")
+        npos = table.shape[0]
+    q = torch.empty(T, nq, dtype=torch.float32, device=proj.device)
+    lib().rope_bias_cache(proj.data_ptr(), proj.stride(0), int(off_q), int(off_k), int(off_v), _ptr(bias),
+                          positions.data_ptr(), _ptr(table) if rot else 0, npos, int(rot), q.data_ptr(),
+                          k_cache.data_ptr(), v_cache.data_ptr(), slots.data_ptr(), T, heads, kv_heads, dim, vdim,
+                          _dt(proj, "proj"), _stream())
+    return q
+
+
+def sink_attn(q, k_cache, v_cache, block_tables, cu, ctx_lens, heads, kv_heads, dim, vdim, scale, softcap,
+              all_groups):
+    T = q.shape[0]
+    _rows(q, "q", heads * dim, torch.float32)
+    _check(q.is_contiguous(), "q contiguous")
+    B = cu.numel() - 1
+    _i32(cu, "cu")
+    _i32(ctx_lens, "ctx_lens", B)
+    _i32(block_tables, "block_tables")
+    _check(block_tables.dim() == 2 and block_tables.shape[0] >= B, "block tables [B, blocks]")
+    _check(k_cache.is_contiguous() and v_cache.is_contiguous() and k_cache.dtype == v_cache.dtype
+           and k_cache.dim() == 3 and k_cache.shape[2] == kv_heads * dim and v_cache.shape[2] == kv_heads * vdim
+           and k_cache.shape[:2] == v_cache.shape[:2], "k / v cache [blocks, block_size, kv_heads * dim | vdim]")
+    R = kv_heads * vdim if all_groups else vdim
+    out = torch.empty(T, heads, R, dtype=torch.float32, device=q.device)
+    lib().sink_attn(q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), block_tables.data_ptr(),
+                    block_tables.shape[1], cu.data_ptr(), ctx_lens.data_ptr(), out.data_ptr(), T, B, heads, kv_heads,
+                    dim, vdim, k_cache.shape[1], float(scale), float(softcap or 0.0), int(bool(all_groups)),
+                    _dt(k_cache, "k cache"), _stream())
+    return out
+
+
+def talk_mix(O, talk, c, heads, kv_heads, vdim, out=None, out_dtype=None):
+    T = O.shape[0]
+    R = kv_heads * vdim if talk is not None else vdim
+    _check(O.dtype == torch.float32 and O.is_contiguous() and tuple(O.shape[1:]) == (heads, R), "O fp32 [T, heads, R]")
+    if talk is not None:
+        _f32c(talk, "talk")
+        _check(talk.numel() == heads * heads, "talk [heads, heads]")
+    if out is None:
+        out = torch.empty(T, heads * vdim, dtype=out_dtype, device=O.device)
+    _rows(out, "out", heads * vdim)
+    lib().talk_mix(O.data_ptr(), _ptr(talk), float(c), out.data_ptr(), out.stride(0), T, heads, kv_heads, vdim,
+                   _dt(out, "out"), _stream())
+    return out

@@ -579,3 +579,228 @@ def moe_experts(h: torch.Tensor, idx: torch.Tensor, wts: torch.Tensor, gate: tor
     if shared is not None:
         out += shared.float()
     return out
+
+
+# ----------------------------------- residual streams / convolution tails / matrix-state recurrences / sink attention
+def _seq_rows(cu, ctx_lens):
+    """(b, first row, rows, first position) of every sequence of a step with rows."""
+    cu_l, cl = cu.tolist(), ctx_lens.tolist()
+    return [(b, cu_l[b], cu_l[b + 1] - cu_l[b], cl[b] - (cu_l[b + 1] - cu_l[b])) for b in range(len(cu_l) - 1)
+            if cu_l[b + 1] > cu_l[b] and cl[b] > 0]
+
+
+def embed_streams(ids, positions, table, pos_table, streams: int) -> torch.Tensor:
+    """fp32 [streams, T, W]: every stream starts as table[ids] (+ pos_table[positions])."""
+    x = table[ids.clamp(0, table.shape[0] - 1)].float()
+    if pos_table is not None:
+        x = x + pos_table[positions.clamp(0, pos_table.shape[0] - 1)].float()
+    return x.unsqueeze(0).repeat(streams, 1, 1).contiguous()
+
+
+def stream_add_norm(x, y, mix, outw, c: float, inw, w, eps: float, rms: bool, out_dtype):
+    """x fp32 [S, T, W], updated in place when ``y`` is given: x_s <- sum_r mix[r, s] x_r + c * outw[s] * y.
+    With ``w``: returns norm(sum_s inw[s] x_s) * w in ``out_dtype`` (inw None: the plain sum; rms False: mean
+    subtracted, variance = mean squared deviation)."""
+    if y is not None:
+        x.copy_(torch.einsum("rs,rtw->stw", mix, x) + (c * outw)[:, None, None] * y.float()[None])
+    if w is None:
+        return None
+    u = x.sum(0) if inw is None else torch.einsum("s,stw->tw", inw, x)
+    if not rms:
+        u = u - u.mean(-1, keepdim=True)
+    return (u * torch.rsqrt(u.pow(2).mean(-1, keepdim=True) + eps) * w.float()).to(out_dtype)
+
+
+def causal_conv(x, w, state, cu, ctx_lens, state_slots, residual: bool, silu: bool, out_dtype):
+    """Per-channel causal convolution over time of x [T, C] with w [C, taps] (last column: the current row), each
+    sequence continuing from the taps - 1 inputs in its state slot (state fp32 [slots, taps - 1, C], renewed here;
+    a portion starting at position 0 reads zeros). ``residual`` adds x itself; ``silu`` applies x * sigmoid(x)."""
+    T, C = x.shape
+    taps = w.shape[1]
+    R = taps - 1
+    out = torch.zeros(T, C, dtype=torch.float32)
+    wf = w.float()
+    slots = state_slots.tolist()
+    for b, t0, q, p0 in _seq_rows(cu, ctx_lens):
+        cur = x[t0:t0 + q].float()
+        if R:
+            tail = state[slots[b]].clone() if p0 > 0 else torch.zeros(R, C)
+            if p0 < R:
+                tail[:R - p0] = 0
+            full = torch.cat([tail, cur], 0)
+            state[slots[b]] = full[-R:]
+        else:
+            full = cur
+        y = sum(wf[:, k] * full[k:k + q] for k in range(taps))
+        if residual:
+            y = y + cur
+        out[t0:t0 + q] = y
+    if silu:
+        out = out * torch.sigmoid(out)
+    return out.to(out_dtype)
+
+
+def gated_group_norm(o, gate, w, eps: float, act: str, c: float, out=None, out_dtype=None):
+    """o fp32 [T, groups * n] divided per group of n = len(w) by its root mean square, times w, times act(gate)
+    (``sigmoid`` or ``silu``), times c; written to ``out`` (a [T, groups * n] view) when given."""
+    T, N = o.shape
+    n = w.numel()
+    og = o.float().view(T, N // n, n)
+    g = gate.float()
+    a = torch.sigmoid(g) if act == "sigmoid" else g * torch.sigmoid(g)
+    y = (og * torch.rsqrt(og.pow(2).mean(-1, keepdim=True) + eps) * w.float()).view(T, N) * a * c
+    if out is not None:
+        out.copy_(y)
+        return out
+    return y.to(out_dtype)
+
+
+def glu_act(gu, F_: int, act: str):
+    """act(gu[:, :F]) * gu[:, F:2F]; act ``gelu_tanh`` or ``silu``."""
+    g, u = gu[:, :F_].float(), gu[:, F_:2 * F_].float()
+    a = torch.nn.functional.gelu(g, approximate="tanh") if act == "gelu_tanh" else g * torch.sigmoid(g)
+    return (a * u).to(gu.dtype)
+
+
+def decay_recurrence(q, k, v, decay, state, cu, ctx_lens, state_slots, heads: int, dim: int, vdim: int,
+                     silu_in: bool = True):
+    """Per head S <- decay_h S + k v^T, o = S^T q over each sequence's rows, S fp32 [slots, heads, dim, vdim]
+    carried in the sequence's slot (zero when the portion starts at position 0). Returns fp32 [T, heads * vdim]."""
+    T = q.shape[0]
+    out = torch.zeros(T, heads * vdim, dtype=torch.float32)
+    slots = state_slots.tolist()
+
+    def pre(t):
+        t = t.float()
+        return t * torch.sigmoid(t) if silu_in else t
+    for b, t0, n, p0 in _seq_rows(cu, ctx_lens):
+        S = state[slots[b]].clone() if p0 > 0 else torch.zeros(heads, dim, vdim)
+        qq = pre(q[t0:t0 + n]).view(n, heads, dim)
+        kk = pre(k[t0:t0 + n]).view(n, heads, dim)
+        vv = pre(v[t0:t0 + n]).view(n, heads, vdim)
+        for j in range(n):
+            S = decay[:, None, None] * S + kk[j, :, :, None] * vv[j, :, None, :]
+            out[t0 + j] = torch.einsum("hdv,hd->hv", S, qq[j]).reshape(-1)
+        state[slots[b]] = S
+    return out
+
+
+def delta_recurrence(q, k, v, a, b_, A_log, dt_bias, state, cu, ctx_lens, state_slots, heads: int, kv_heads: int,
+                     dim: int, vdim: int):
+    """Gated delta rule per head: S <- g S; u = beta (v - S^T k); S <- S + k u^T; o = S^T q, with k and q made unit
+    vectors (1e-6 inside the root), q also divided by sqrt(dim), beta = sigmoid(b), g = exp(-exp(A_log)
+    softplus(a + dt_bias)). q, k [T, kv_heads * dim], v [T, heads * vdim], a, b_ [T, heads]. fp32 out."""
+    T = q.shape[0]
+    rep = heads // kv_heads
+    out = torch.zeros(T, heads * vdim, dtype=torch.float32)
+    slots = state_slots.tolist()
+    for b, t0, n, p0 in _seq_rows(cu, ctx_lens):
+        S = state[slots[b]].clone() if p0 > 0 else torch.zeros(heads, dim, vdim)
+        qq = q[t0:t0 + n].float().view(n, kv_heads, dim)
+        kk = k[t0:t0 + n].float().view(n, kv_heads, dim)
+        qq = (qq * torch.rsqrt(qq.pow(2).sum(-1, keepdim=True) + 1e-6) * dim ** -0.5).repeat_interleave(rep, 1)
+        kk = (kk * torch.rsqrt(kk.pow(2).sum(-1, keepdim=True) + 1e-6)).repeat_interleave(rep, 1)
+        vv = v[t0:t0 + n].float().view(n, heads, vdim)
+        beta = torch.sigmoid(b_[t0:t0 + n].float())
+        g = torch.exp(-torch.exp(A_log.float()) * torch.nn.functional.softplus(a[t0:t0 + n].float() + dt_bias.float()))
+        for j in range(n):
+            S = g[j][:, None, None] * S
+            u = beta[j][:, None] * (vv[j] - torch.einsum("hdv,hd->hv", S, kk[j]))
+            S = S + kk[j][:, :, None] * u[:, None, :]
+            out[t0 + j] = torch.einsum("hdv,hd->hv", S, qq[j]).reshape(-1)
+        state[slots[b]] = S
+    return out
+
+
+def rope_angle_table(npos: int, dims: int, base: float, scaling=None) -> torch.Tensor:
+    """fp32 [npos, dims / 2, 2] = (cos, sin) of position * f_i, f_i = base^(-2 i / dims). ``scaling`` = (factor,
+    original, fast, slow): frequencies between the two turn counts are blended towards f_i / factor (YaRN) and both
+    cos and sin are multiplied by 0.1 ln(factor) + 1. Angles are formed in float64 and rounded once."""
+    half = dims // 2
+    f = torch.tensor([base ** (-2.0 * i / dims) for i in range(half)], dtype=torch.float64)
+    amp = 1.0
+    if scaling is not None:
+        factor, original, fast, slow = scaling
+
+        def turn_dim(turns):
+            return dims * math.log(original / (2.0 * math.pi * turns)) / (2.0 * math.log(base))
+        lo = max(math.floor(turn_dim(fast)), 0)
+        hi = min(math.ceil(turn_dim(slow)), dims - 1)
+        ramp = ((torch.arange(half, dtype=torch.float64) - lo) / max(hi - lo, 0.001)).clamp(0, 1)
+        f = f / factor * ramp + f * (1 - ramp)
+        amp = 0.1 * math.log(factor) + 1.0
+    ang = torch.arange(npos, dtype=torch.float64)[:, None] * f[None, :]
+    return torch.stack([torch.cos(ang) * amp, torch.sin(ang) * amp], -1).float().contiguous()
+
+
+def rope_bias_cache(proj, off_q: int, off_k: int, off_v: int, bias, positions, table, rot: int, k_cache, v_cache,
+                    slots, heads: int, kv_heads: int, dim: int, vdim: int):
+    """From the projection rows: q (+ bias) and k (+ bias) with their first ``rot`` dimensions per head turned by
+    ``table`` (i paired with i + rot / 2), v (+ bias). Returns q fp32 [T, heads * dim]; k / v go into the paged
+    caches [blocks, block_size, kv_heads * dim | kv_heads * vdim] at ``slots`` (< 0: not cached)."""
+    T = proj.shape[0]
+    nq, nk, nv = heads * dim, kv_heads * dim, kv_heads * vdim
+    q, k, v = (proj[:, o:o + n].float() for o, n in ((off_q, nq), (off_k, nk), (off_v, nv)))
+    if bias is not None:
+        bf = bias.float()
+        q, k, v = q + bf[:nq], k + bf[nq:nq + nk], v + bf[nq + nk:]
+    half = rot // 2
+    if half:
+        cs = table[positions.clamp(0, table.shape[0] - 1)]  # [T, half, 2]
+        c, s = cs[:, None, :, 0], cs[:, None, :, 1]
+
+        def turn(x, n):
+            x = x.view(T, n, dim)
+            a, b = x[..., :half], x[..., half:rot]
+            return torch.cat([a * c - b * s, b * c + a * s, x[..., rot:]], -1).reshape(T, n * dim)
+        q, k = turn(q, heads), turn(k, kv_heads)
+    keep = slots >= 0
+    k_cache.view(-1, nk)[slots[keep]] = k[keep].to(k_cache.dtype)
+    v_cache.view(-1, nv)[slots[keep]] = v[keep].to(v_cache.dtype)
+    return q.contiguous()
+
+
+def sink_attn(q, k_cache, v_cache, block_tables, cu, ctx_lens, heads: int, kv_heads: int, dim: int, vdim: int,
+              scale: float, softcap: float, all_groups: bool):
+    """Causal attention of every row over its sequence's cached keys with a sink in the softmax denominator
+    (p_j = exp(s_j) / (1 + sum exp(s))) and optionally soft-capped scores. Returns fp32 [T, heads, R]: head h's
+    weights applied to the value rows of every group side by side (``all_groups``, R = kv_heads * vdim) or of its
+    own group only (R = vdim)."""
+    T = q.shape[0]
+    bs = k_cache.shape[1]
+    rep = heads // kv_heads
+    R = kv_heads * vdim if all_groups else vdim
+    out = torch.zeros(T, heads, R, dtype=torch.float32)
+    for b, t0, n, p0 in _seq_rows(cu, ctx_lens):
+        L = p0 + n
+        blocks = block_tables[b, : -(-L // bs)].long()
+        K = k_cache[blocks].reshape(-1, kv_heads, dim)[:L].float()
+        V = v_cache[blocks].reshape(-1, kv_heads, vdim)[:L].float()
+        qq = q[t0:t0 + n].view(n, heads, dim).float()
+        s = torch.einsum("nhd,lhd->hnl", qq, K.repeat_interleave(rep, 1)) * scale
+        if softcap:
+            s = softcap * torch.tanh(s / softcap)
+        vis = torch.arange(L)[None, :] <= (p0 + torch.arange(n))[:, None]
+        e = torch.exp(s - s.amax(-1, keepdim=True).clamp(min=0)) * vis
+        p = e / (torch.exp(-s.amax(-1, keepdim=True).clamp(min=0)) + e.sum(-1, keepdim=True))
+        if all_groups:
+            out[t0:t0 + n] = torch.einsum("hnl,lr->nhr", p, V.reshape(L, R))
+        else:
+            out[t0:t0 + n] = torch.einsum("hnl,lhv->nhv", p, V.repeat_interleave(rep, 1))
+    return out
+
+
+def talk_mix(O, talk, c: float, heads: int, kv_heads: int, vdim: int, out=None, out_dtype=None):
+    """y[t, h, :] = c * sum_h' talk[h, h'] O[t, h', group(h) part] (talk None: c * O). [T, heads * vdim]."""
+    T = O.shape[0]
+    rep = heads // kv_heads
+    if talk is None:
+        y = O.reshape(T, heads * vdim) * c
+    else:
+        Og = O.view(T, heads, kv_heads, vdim)
+        grp = torch.arange(heads) // rep
+        y = torch.einsum("hg,tghv->thv", talk.float(), Og[:, :, grp, :]).reshape(T, heads * vdim) * c
+    if out is not None:
+        out.copy_(y)
+        return out
+    return y.to(out_dtype)
