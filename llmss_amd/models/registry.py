@@ -21,7 +21,7 @@ from ..parallel.dist import TPGroup
 from .config import ModelConfig
 from .decoder import StepInput
 from .layered import create_model
-from .weights import load_hf_weights, load_timisun_weights
+from .weights import load_babotar_weights, load_hf_weights, load_timisun_weights
 
 
 @dataclass
@@ -32,9 +32,10 @@ class CausalLMOutput:
 
 
 class PagedPast:
-    def __init__(self, lens, blocks):
+    def __init__(self, lens, blocks, state=None):
         self.lens = lens  # tokens cached per row
         self.blocks = blocks  # list of block-id lists per row
+        self.state = state  # models with per-sequence state: the state slot of each row (-1: none yet)
 
 
 class CausalLM:
@@ -50,19 +51,23 @@ class CausalLM:
     embeddings; by default a row's tokens take consecutive positions after its cached ones.
     """
 
-    def __init__(self, config, weights, max_blocks: int = 4096, block_size: int = 16):
+    def __init__(self, config, weights, max_blocks: int = 4096, block_size: int = 16, max_seqs: int = 16):
         cfg = config if isinstance(config, ModelConfig) else ModelConfig.from_hf_dict(config.to_dict())
         tp = getattr(weights, "tp", None) or TPGroup()
-        if cfg.layer_specs:  # per-layer designs (Timisun)
-            w = load_timisun_weights(cfg, weights.reader, device=weights.device, dtype=weights.dtype)
+        if cfg.layer_specs:  # per-layer designs (Timisun, Babotar)
+            load = load_babotar_weights if cfg.model_type == "babotar" else load_timisun_weights
+            w = load(cfg, weights.reader, device=weights.device, dtype=weights.dtype)
         else:
             w = load_hf_weights(cfg, weights.reader, tp.size, tp.rank, device=weights.device, dtype=weights.dtype)
         self.model = create_model(cfg, w, tp)
         self.config = cfg
         self.block_size = block_size
         self.max_blocks = max_blocks
-        self.kv = self.model.allocate_kv_cache(max_blocks, block_size)
+        self.stateful = bool(getattr(self.model, "needs_state", False))
+        self.kv = (self.model.allocate_kv_cache(max_blocks, block_size, num_slots=max_seqs) if self.stateful
+                   else self.model.allocate_kv_cache(max_blocks, block_size))
         self._free = list(range(max_blocks - 1, -1, -1))
+        self._free_state = list(range(max_seqs - 1, -1, -1))
 
     def eval(self):
         return self
@@ -77,6 +82,9 @@ class CausalLM:
             for b in past.blocks:
                 self._free.extend(b)
             past.blocks = [[] for _ in past.blocks]
+            if past.state is not None:
+                self._free_state.extend(s for s in past.state if s >= 0)
+                past.state = [-1] * len(past.state)
 
     @torch.no_grad()
     def __call__(self, input_ids, past_key_values: Optional[PagedPast] = None, use_cache: bool = False,
@@ -93,7 +101,7 @@ class CausalLM:
         dev = self.model.device
         B, S = input_ids.shape
         bs = self.block_size
-        past = past_key_values or PagedPast([0] * B, [[] for _ in range(B)])
+        past = past_key_values or PagedPast([0] * B, [[] for _ in range(B)], [-1] * B if self.stateful else None)
         if attention_mask is not None:
             am = attention_mask.to("cpu").bool()
             if am.shape[0] != B or am.shape[1] < S:
@@ -117,9 +125,13 @@ class CausalLM:
             needs = [max(0, -(-(start + len(cols)) // bs) - len(past.blocks[b])) for b, cols, start in order]
             if sum(needs) > len(self._free):
                 raise RuntimeError("CausalLM: KV pool exhausted")
+            if self.stateful and sum(past.state[b] < 0 for b, _, _ in order) > len(self._free_state):
+                raise RuntimeError("CausalLM: no free state slot")
             for (b, _, _), need in zip(order, needs):
                 if need:
                     past.blocks[b].extend(self._alloc(need))
+                if self.stateful and past.state[b] < 0:
+                    past.state[b] = self._free_state.pop()
             tok, pos, slots, qlens, ctx, bt_rows = [], [], [], [], [], []
             for b, cols, start in order:
                 n = len(cols)
@@ -145,10 +157,12 @@ class CausalLM:
                             torch.tensor(slots, dtype=torch.int64, device=dev), cu_seqlens=cu.to(dev),
                             max_seqlen=int(qt[nd:].max()) if ext else 0, block_tables=bt.to(dev),
                             ctx_lens=torch.tensor(ctx, dtype=torch.int32, device=dev), max_ctx=maxb * bs,
-                            num_decode=nd, has_prefix=has_prefix)
+                            num_decode=nd, has_prefix=has_prefix,
+                            state_slots=torch.tensor([past.state[b] for b, _, _ in order], dtype=torch.int32,
+                                                     device=dev) if self.stateful else None)
             if kind == "extend" and not ext:  # decodes only
                 inp = StepInput("decode", inp.input_ids, inp.positions, inp.slots, block_tables=inp.block_tables,
-                                ctx_lens=inp.ctx_lens, max_ctx=inp.max_ctx)
+                                ctx_lens=inp.ctx_lens, max_ctx=inp.max_ctx, state_slots=inp.state_slots)
             logits = self.model.logits(self.model.hidden_states(inp, self.kv)).float()
             r0 = 0
             for (b, cols, start), n in zip(order, qlens):
@@ -256,5 +270,11 @@ class TimisunForCausalLM(_FamilyLM):
     model_type = "timisun"
 
 
+class BabotarForCausalLM(_FamilyLM):
+    """Per-layer design: sink attention beside a gated delta rule, decay linear attention, residual streams with
+    learned connections (models/layered.py)."""
+    model_type = "babotar"
+
+
 MODEL_REGISTRY = {c.model_type: c for c in (GPT2LMHeadModel, GPTJForCausalLM, GPTBigCodeForCausalLM,
-                                            LlamaForCausalLM, TimisunForCausalLM)}
+                                            LlamaForCausalLM, TimisunForCausalLM, BabotarForCausalLM)}

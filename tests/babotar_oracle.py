@@ -207,3 +207,10 @@ def forward(cfg, W, tokens):
         after.append(sum(xs))
     x = layer_norm(sum(xs), W["final.norm"], eps)
     return x @ W["head"].T, torch.stack(after)
+
+
+def greedy(cfg, W, prompt, n):
+    seq = list(prompt)
+    for _ in range(n):
+        seq.append(int(forward(cfg, W, seq)[0][-1].argmax()))
+    return seq[len(prompt):]
