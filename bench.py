@@ -78,7 +78,22 @@ def main():
                          "the Llama family at equal size (bench/timisun_compare.py), sizes by name, one GPU")
     ap.add_argument("--timisun-rounds", type=int, default=2)
     ap.add_argument("--timisun-kinds", default="timisun,dense", help="which of the two models --timisun runs")
+    ap.add_argument("--babotar", nargs="?", const="w1024,w2048,w4096", default="",
+                    help="instead of the headline workload: prefill / decode throughput of the Babotar design beside "
+                         "the Llama family at equal size (bench/babotar_compare.py), sizes by name, one GPU")
+    ap.add_argument("--babotar-kinds", default="babotar,dense", help="which of the two models --babotar runs")
     args = ap.parse_args()
+
+    if args.babotar:
+        sys.path.insert(0, os.path.join(ROOT, "bench"))
+        import babotar_compare
+
+        res = babotar_compare.run(args.babotar.split(","), args.batch_per_gpu, args.prompt_len, args.gen_len,
+                                  args.timisun_rounds,
+                                  lambda m: print(f"[bench] {m}", file=sys.stderr, flush=True),
+                                  kinds=tuple(args.babotar_kinds.split(",")))
+        print(json.dumps(res), flush=True)
+        return
 
     if args.timisun:
         sys.path.insert(0, os.path.join(ROOT, "bench"))

@@ -74,38 +74,43 @@ void launch_rope_bias_cache(const void* proj, int64_t ldp, int off_q, int off_k,
   HIP_CHECK_LAUNCH();
 }
 
-// Workgroup: one row t, one key group g, NW of its query heads (a wave each). Grid (T, G * chunks of heads, chunks
-// of value columns). A block of KB keys of group g is staged in LDS for all waves; a wave scores it with lanes over
-// keys, updates its online softmax and accumulates over value columns (lanes over columns, NR registers per lane),
-// reading value rows from the cache. Value columns v0 .. v0 + RV - 1 of the key's whole value row [G * vdim]
-// (all = 1) or of group g's part (all = 0). out [T, H, RVtot] fp32.
-template <typename T, int NR>
+// Vector kernel (any shape, either storage type; single decoded rows and what the matrix-core kernel below does not
+// take). Workgroup: one row t, one key group g, up to NWT of its query heads. Grid (T, G * chunks of heads, chunks of
+// value columns). A block of KB keys of group g is staged in LDS once; wave w scores it for head w with lanes over
+// keys, updates that head's online softmax and leaves the weights in LDS. Then the waves split the VALUE COLUMNS
+// between them: wave w accumulates its slice of columns for ALL heads of the workgroup, so a value row is read once
+// per workgroup, straight from the cache, 8 or 16 keys' loads in flight at a time. Value columns v0 .. v0 + RV - 1 of
+// the key's whole value row [G * vdim] (all = 1) or of group g's part (all = 0). out [T, H, RVtot] fp32.
+template <typename T, int NWT, int NR2, bool WORDS>
 __global__ void sink_attn_kernel(const float* __restrict__ q, const T* __restrict__ kc, const T* __restrict__ vc,
                                  const int* __restrict__ bt, int maxb, const int* __restrict__ cu,
                                  const int* __restrict__ ctx, float* __restrict__ out, int B, int H, int G, int dim,
                                  int vdim, int bs, float scale, float cap, int all, int KB, int Dp, int hchunks,
                                  int RVchunk) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-  const int NW = blockDim.x >> 6;
   T* tile = reinterpret_cast<T*>(smem);
   float* qs = reinterpret_cast<float*>(smem + (((size_t)KB * Dp * sizeof(T) + 15) & ~(size_t)15));
-  float* ps = qs + (size_t)NW * dim;
+  float* ps = qs + (size_t)NWT * dim;      // [NWT][KB] weights of the current block of keys
+  float* hs = ps + (size_t)NWT * KB;       // [NWT][2]: the block's rescale factor, the final denominator
+  // [KB] cache row of each staged key, on the next 8-byte boundary
+  int64_t* srow = reinterpret_cast<int64_t*>((reinterpret_cast<uintptr_t>(hs + 2 * NWT) + 7) & ~(uintptr_t)7);
   const int t = blockIdx.x, wv = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int rep = H / G;
   const int g = blockIdx.y / hchunks;
-  const int hl = (blockIdx.y % hchunks) * NW + wv;
-  const bool live = hl < rep;
-  const int h = g * rep + hl;
+  const int hl0 = (blockIdx.y % hchunks) * NWT;
+  const bool live = hl0 + wv < rep;  // this wave scores a head
+  const int h = g * rep + hl0 + wv;
   const int RVtot = all ? G * vdim : vdim;
   const int v0 = blockIdx.z * RVchunk;
   const int RV = min(RVchunk, RVtot - v0);
   const int64_t vrow = (int64_t)G * vdim;
   const int voff = (all ? 0 : g * vdim) + v0;
+  const int cs = NR2 * 64;  // columns per wave
+  constexpr int VK = NR2 >= 4 ? 8 : 16;  // keys whose value loads are in flight together
   const RowSeq r = row_seq(cu, ctx, B, t);
-  float* o = out + ((int64_t)t * H + h) * RVtot + v0;
   if (r.pos < 0) {
-    if (live)
-      for (int i = lane; i < RV; i += 64) o[i] = 0.f;
+    for (int hh = 0; hh < NWT && hl0 + hh < rep; ++hh)
+      for (int i = threadIdx.x; i < RV; i += blockDim.x) out[((int64_t)t * H + g * rep + hl0 + hh) * RVtot + v0 + i] = 0.f;
     return;
   }
   float* qw = qs + (size_t)wv * dim;
@@ -114,29 +119,55 @@ __global__ void sink_attn_kernel(const float* __restrict__ q, const T* __restric
     const float* qsrc = q + ((int64_t)t * H + h) * dim;
     for (int d = lane; d < dim; d += 64) qw[d] = qsrc[d] * scale;
   }
-  float acc[NR];
+  float acc[NWT][NR2];
 #pragma unroll
-  for (int i = 0; i < NR; ++i) acc[i] = 0.f;
+  for (int hh = 0; hh < NWT; ++hh)
+#pragma unroll
+    for (int i = 0; i < NR2; ++i) acc[hh][i] = 0.f;
   float m = 0.f, l = 1.f;  // the sink: score 0, weight exp(0 - m), no value
   const float icap = cap > 0.f ? 1.0f / cap : 0.f;
   const int* btr = bt + (int64_t)r.b * maxb;
+  const int c0 = wv * cs + lane;  // this lane's first column within the chunk
   for (int j0 = 0; j0 <= r.pos; j0 += KB) {
     const int nk = min(KB, r.pos - j0 + 1);
     __syncthreads();
-    for (int kk = wv; kk < nk; kk += NW) {
+    for (int kk = threadIdx.x; kk < nk; kk += blockDim.x) {
       const int j = j0 + kk;
-      const int64_t slot = (int64_t)btr[j / bs] * bs + j % bs;
-      const T* src = kc + (slot * G + g) * dim;
-      T* dst = tile + (size_t)kk * Dp;
-      for (int d = lane; d < dim; d += 64) dst[d] = src[d];
+      srow[kk] = (int64_t)btr[j / bs] * bs + j % bs;
+    }
+    __syncthreads();
+    if (WORDS) {  // rows copied as 4-byte words by all threads, several loads in flight per thread
+      const int wpr = dim * (int)sizeof(T) / 4, ldw = Dp * (int)sizeof(T) / 4;
+      const unsigned* kw = reinterpret_cast<const unsigned*>(kc);
+      unsigned* tw = reinterpret_cast<unsigned*>(tile);
+#pragma unroll 4
+      for (int e = threadIdx.x; e < nk * wpr; e += blockDim.x) {
+        const int kk = e / wpr, wd = e - kk * wpr;
+        tw[(size_t)kk * ldw + wd] = kw[(srow[kk] * G + g) * wpr + wd];
+      }
+    } else {
+      for (int e = threadIdx.x; e < nk * dim; e += blockDim.x) {
+        const int kk = e / dim, d = e - kk * dim;
+        tile[(size_t)kk * Dp + d] = kc[(srow[kk] * G + g) * dim + d];
+      }
     }
     __syncthreads();
     if (live) {
       float s = -INFINITY;
       if (lane < nk) {
         const T* row = tile + (size_t)lane * Dp;
-        float d_ = 0.f;
-        for (int d = 0; d < dim; ++d) d_ = fmaf(qw[d], El<T>::ld(row + d), d_);
+        float d_ = 0.f, d2 = 0.f;
+        if (WORDS && sizeof(T) == 2) {  // two keys' numbers per LDS read
+          const unsigned* rw = reinterpret_cast<const unsigned*>(row);
+          for (int w2 = 0; w2 < dim / 2; ++w2) {
+            const unsigned u = rw[w2];
+            d_ = fmaf(qw[2 * w2], __uint_as_float(u << 16), d_);
+            d2 = fmaf(qw[2 * w2 + 1], __uint_as_float(u & 0xffff0000u), d2);
+          }
+          d_ += d2;
+        } else {
+          for (int d = 0; d < dim; ++d) d_ = fmaf(qw[d], El<T>::ld(row + d), d_);
+        }
         s = cap > 0.f ? cap * tanhf(d_ * icap) : d_;
       }
       const float m_new = fmaxf(m, warp_max(s));
@@ -145,30 +176,54 @@ __global__ void sink_attn_kernel(const float* __restrict__ q, const T* __restric
       l = l * alpha + warp_sum(pj);
       m = m_new;
       if (lane < KB) p[lane] = pj;
-#pragma unroll
-      for (int i = 0; i < NR; ++i) acc[i] *= alpha;
+      if (lane == 0) hs[2 * wv] = alpha;
+    } else {
+      if (lane < KB) p[lane] = 0.f;
+      if (lane == 0) hs[2 * wv] = 1.f;
     }
-    __syncthreads();
-    if (live) {
-      for (int kk = 0; kk < nk; ++kk) {
-        const float pj = p[kk];
-        const int j = j0 + kk;
-        const int64_t slot = (int64_t)btr[j / bs] * bs + j % bs;
-        const T* row = vc + slot * vrow + voff;
+    __syncthreads();  // weights, rescale factors and cache rows visible to every wave
 #pragma unroll
-        for (int i = 0; i < NR; ++i) {
-          const int c = lane + 64 * i;
-          if (c < RV) acc[i] = fmaf(pj, El<T>::ld(row + c), acc[i]);
+    for (int hh = 0; hh < NWT; ++hh) {
+      const float al = hs[2 * hh];
+#pragma unroll
+      for (int i = 0; i < NR2; ++i) acc[hh][i] *= al;
+    }
+    for (int k0 = 0; k0 < nk; k0 += VK) {
+      float vv[VK][NR2];
+#pragma unroll
+      for (int j = 0; j < VK; ++j) {
+        const T* row = vc + srow[min(k0 + j, nk - 1)] * vrow + voff;
+#pragma unroll
+        for (int i = 0; i < NR2; ++i) {
+          const int c = c0 + 64 * i;
+          vv[j][i] = c < RV ? El<T>::ld(row + c) : 0.f;
+        }
+      }
+#pragma unroll
+      for (int j = 0; j < VK; ++j) {
+        if (k0 + j < nk) {
+#pragma unroll
+          for (int hh = 0; hh < NWT; ++hh) {
+            const float pj = ps[hh * KB + k0 + j];
+#pragma unroll
+            for (int i = 0; i < NR2; ++i) acc[hh][i] = fmaf(pj, vv[j][i], acc[hh][i]);
+          }
         }
       }
     }
   }
-  if (live) {
-    const float inv = 1.0f / l;
+  if (lane == 0) hs[2 * wv + 1] = l;
+  __syncthreads();
 #pragma unroll
-    for (int i = 0; i < NR; ++i) {
-      const int c = lane + 64 * i;
-      if (c < RV) o[c] = acc[i] * inv;
+  for (int hh = 0; hh < NWT; ++hh) {
+    if (hl0 + hh < rep) {
+      const float inv = 1.0f / hs[2 * hh + 1];
+      float* o = out + ((int64_t)t * H + g * rep + hl0 + hh) * RVtot + v0;
+#pragma unroll
+      for (int i = 0; i < NR2; ++i) {
+        const int c = c0 + 64 * i;
+        if (c < RV) o[c] = acc[hh][i] * inv;
+      }
     }
   }
 }
@@ -178,7 +233,7 @@ static void sink_attn_t(const void* q, const void* kc, const void* vc, const voi
                         const void* ctx, void* out, int T_, int B, int H, int G, int dim, int vdim, int bs,
                         float scale, float cap, int all, hipStream_t st) {
   const int rep = H / G;
-  const int NW = std::min(rep, 8);
+  const int NW = rep >= 8 ? 8 : (rep > 2 ? 4 : rep);  // waves = heads per workgroup: 1, 2, 4 or 8
   const int hchunks = (rep + NW - 1) / NW;
   int Dp;  // key row stride in LDS: an odd number of 4-byte words (lanes score neighbouring keys)
   if (sizeof(T) == 2) {
@@ -188,25 +243,46 @@ static void sink_attn_t(const void* q, const void* kc, const void* vc, const voi
     Dp = dim | 1;
   }
   int KB = 64;
-  auto bytes = [&](int kb) { return (((size_t)kb * Dp * sizeof(T) + 15) & ~(size_t)15) + (size_t)NW * (dim + kb) * 4; };
-  while (KB > 4 && bytes(KB) > 60 * 1024) KB >>= 1;
+  auto bytes = [&](int kb) {
+    return (((size_t)kb * Dp * sizeof(T) + 15) & ~(size_t)15) + (size_t)NW * (dim + kb + 2) * 4 + (size_t)kb * 8 + 16;
+  };
+  while (KB > 8 && bytes(KB) > 60 * 1024) KB >>= 1;
   if (bytes(KB) > 60 * 1024) throw std::runtime_error("sink attention: head dimension too large for LDS");
   const int RVtot = all ? G * vdim : vdim;
-  const int RVchunk = std::min(RVtot, 512);
+  // columns per workgroup: NW waves x NR2 x 64, NR2 in {1, 2, 4} with at most 16 accumulators per lane
+  int nr2 = 1;
+  while (nr2 < 4 && NW * nr2 * 2 <= 16 && NW * nr2 * 64 < RVtot) nr2 <<= 1;
+  const int RVchunk = std::min(RVtot, NW * nr2 * 64);
   const int zch = (RVtot + RVchunk - 1) / RVchunk;
   if (G * hchunks > 65535 || zch > 65535) throw std::runtime_error("sink attention: too many heads");
   dim3 g(T_, G * hchunks, zch);
-  const int nr = (RVchunk + 63) / 64;
-#define LAUNCH_SA(NR_)                                                                                              \
-  sink_attn_kernel<T, NR_><<<g, NW * 64, bytes(KB), st>>>((const float*)q, (const T*)kc, (const T*)vc,              \
-                                                          (const int*)bt, maxb, (const int*)cu, (const int*)ctx,    \
-                                                          (float*)out, B, H, G, dim, vdim, bs, scale, cap, all, KB, \
-                                                          Dp, hchunks, RVchunk)
-  if (nr <= 1) LAUNCH_SA(1);
-  else if (nr <= 2) LAUNCH_SA(2);
-  else if (nr <= 4) LAUNCH_SA(4);
-  else LAUNCH_SA(8);
+  // whole 4-byte words per key row, word-aligned rows: the word copy and the two-numbers-per-read dot product
+  const bool words = (dim * sizeof(T)) % 4 == 0 && ((uintptr_t)kc % 4) == 0;
+#define LAUNCH_SA1(NW_, NR_, WD_)                                                                            \
+  sink_attn_kernel<T, NW_, NR_, WD_><<<g, NW_ * 64, bytes(KB), st>>>(                                        \
+      (const float*)q, (const T*)kc, (const T*)vc, (const int*)bt, maxb, (const int*)cu, (const int*)ctx,    \
+      (float*)out, B, H, G, dim, vdim, bs, scale, cap, all, KB, Dp, hchunks, RVchunk)
+#define LAUNCH_SA(NW_, NR_)               \
+  do {                                    \
+    if (words) LAUNCH_SA1(NW_, NR_, true); \
+    else LAUNCH_SA1(NW_, NR_, false);     \
+  } while (0)
+#define LAUNCH_SA_NR(NW_)                \
+  do {                                   \
+    if (nr2 == 1) LAUNCH_SA(NW_, 1);     \
+    else if (nr2 == 2) LAUNCH_SA(NW_, 2); \
+    else LAUNCH_SA(NW_, 4);              \
+  } while (0)
+  if (NW == 1) LAUNCH_SA_NR(1);
+  else if (NW == 2) LAUNCH_SA_NR(2);
+  else if (NW == 4) LAUNCH_SA_NR(4);
+  else {
+    if (nr2 == 1) LAUNCH_SA(8, 1);
+    else LAUNCH_SA(8, 2);
+  }
+#undef LAUNCH_SA_NR
 #undef LAUNCH_SA
+#undef LAUNCH_SA1
 }
 
 void launch_sink_attn(const void* q, const void* kc, const void* vc, const void* bt, int maxb, const void* cu,
@@ -216,6 +292,222 @@ void launch_sink_attn(const void* q, const void* kc, const void* vc, const void*
   if (G < 1 || H % G) throw std::runtime_error("sink attention: heads must be a multiple of the key/value heads");
   DISPATCH_T(dt, T, (sink_attn_t<T>(q, kc, vc, bt, maxb, cu, ctx, out, T_, B, H, G, dim, vdim, bs, scale, cap, all,
                                     st)));
+  HIP_CHECK_LAUNCH();
+}
+
+// The same attention on the matrix cores, for portions of bf16 prompts (key size 64 or 128, value size a multiple
+// of 8). One workgroup serves one key/value group, GE of its query heads and 64 / GE query rows of one sequence:
+// the 64 "slots" of its four waves enumerate (row, head) pairs, slot s -> row s / GE, head s % GE, so a key tile is
+// staged in LDS once for the whole head group. Per wave (16 slots) the products are the swapped ones,
+//   S^T[key][slot] = K . Q^T   (A = K rows from LDS, B = Q^T fragments in registers)
+//   O^T[c][slot]  += V^T . P^T (A = V^T by transposing LDS reads, B = P^T straight from the S^T accumulators)
+// so a lane owns one slot's softmax row: cap, mask, running maximum (starting at the sink's 0) and sum need two
+// shuffles per tile. The value tile holds VCH = 16 * NVT columns of the key's value row - all groups side by side
+// when the heads' weights are mixed afterwards - and blockIdx.y also enumerates the column chunks.
+template <int DK, int NVT>
+__global__ __launch_bounds__(256, 2) void sink_attn_mfma_kernel(
+    const float* __restrict__ q, const bf16_t* __restrict__ kc, const bf16_t* __restrict__ vc,
+    const int* __restrict__ block_tables, int max_blocks, const int* __restrict__ cu_q, const int* __restrict__ ctx_lens,
+    float* __restrict__ out, int H, int G, int GE, int vdim, int bs, float scale, float cap, int all, int nvch) {
+  constexpr int BKV = 64;
+  constexpr int LDK = DK + 16;
+  constexpr int VCH = NVT * 16;
+  constexpr int LDV = VCH + 16;
+  __shared__ __attribute__((aligned(16))) bf16_t Ks[BKV * LDK];
+  __shared__ __attribute__((aligned(16))) bf16_t Vs[BKV * LDV];
+  const int rep = H / G;
+  const int rows_per_wg = 64 / GE;
+  const int b = blockIdx.z;
+  const int vch = blockIdx.y % nvch, hy = blockIdx.y / nvch;
+  const int kvh = hy / (rep / GE);
+  const int h0 = kvh * rep + (hy % (rep / GE)) * GE;
+  const int t0 = cu_q[b], qlen = cu_q[b + 1] - t0;
+  const int r0 = blockIdx.x * rows_per_wg;
+  if (r0 >= qlen) return;
+  const int p0 = ctx_lens[b] - qlen;
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  const int li = lane & 15, g = lane >> 4;
+  const int slot = w * 16 + li;
+  const int row = r0 + slot / GE, h = h0 + slot % GE;
+  const bool valid = slot < rows_per_wg * GE && row < qlen;
+  const int qpos = p0 + (valid ? row : 0);
+  const int RVtot = all ? G * vdim : vdim;
+  const int v0 = vch * VCH;
+  const int64_t vrow = (int64_t)G * vdim;
+  const int voff = (all ? 0 : kvh * vdim) + v0;
+
+  s16x8 qf[DK / 32];
+  {
+    const float* qp = q + ((int64_t)(t0 + (valid ? row : 0)) * H + (valid ? h : h0)) * DK + 8 * g;
+#pragma unroll
+    for (int ks = 0; ks < DK / 32; ++ks)
+#pragma unroll
+      for (int j = 0; j < 8; ++j) qf[ks][j] = (short)f2bf(qp[32 * ks + j]);
+  }
+  f32x4 o[NVT];
+#pragma unroll
+  for (int i = 0; i < NVT; ++i) o[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+  float m = 0.f, lsum = 1.f;  // the sink: score 0, weight exp(0 - m), no value
+  const float icap = cap > 0.f ? 1.0f / cap : 0.f;
+  const int r_last = min(qlen, r0 + rows_per_wg) - 1;
+  const int kv_end = p0 + r_last + 1;
+  const int wave_qhi = p0 + min(qlen - 1, r0 + (16 * w + 15) / GE);
+  const int* bt = block_tables + (int64_t)b * max_blocks;
+  constexpr int CHK = DK / 8, CHV = VCH / 8;
+  // Software pipeline: the next tile's 16-byte chunks are fetched into registers while this tile is computed from
+  // LDS, and written to LDS after the next barrier, so a tile does not wait a memory round trip behind the last one.
+  static_assert((BKV * CHK) % 256 == 0 && (BKV * CHV) % 256 == 0, "whole 16-byte chunks per thread");
+  constexpr int NCK = BKV * CHK / 256, NCV = BKV * CHV / 256;
+  u16x8 kr[NCK], vr[NCV];
+  auto load_tile = [&](int kv0) {
+#pragma unroll
+    for (int j = 0; j < NCK; ++j) {
+      const int c = threadIdx.x + 256 * j;
+      const int r = c / CHK, ch = c % CHK;
+      const int key = min(kv0 + r, kv_end - 1);
+      const int64_t sl = (int64_t)bt[key / bs] * bs + key % bs;
+      kr[j] = *reinterpret_cast<const u16x8*>(kc + (sl * G + kvh) * DK + ch * 8);
+    }
+#pragma unroll
+    for (int j = 0; j < NCV; ++j) {
+      const int c = threadIdx.x + 256 * j;
+      const int r = c / CHV, ch = c % CHV;
+      const int key = min(kv0 + r, kv_end - 1);
+      const int64_t sl = (int64_t)bt[key / bs] * bs + key % bs;
+      u16x8 val = {0, 0, 0, 0, 0, 0, 0, 0};
+      if (v0 + ch * 8 < RVtot) val = *reinterpret_cast<const u16x8*>(vc + sl * vrow + voff + ch * 8);
+      vr[j] = val;
+    }
+  };
+  auto store_tile = [&]() {
+#pragma unroll
+    for (int j = 0; j < NCK; ++j) {
+      const int c = threadIdx.x + 256 * j;
+      *reinterpret_cast<u16x8*>(&Ks[(c / CHK) * LDK + (c % CHK) * 8]) = kr[j];
+    }
+#pragma unroll
+    for (int j = 0; j < NCV; ++j) {
+      const int c = threadIdx.x + 256 * j;
+      *reinterpret_cast<u16x8*>(&Vs[(c / CHV) * LDV + (c % CHV) * 8]) = vr[j];
+    }
+  };
+  // a wave none of whose slots holds a row (a single decoded row fills part of the first wave) only helps to stage
+  const bool wave_rows = r0 + (16 * w) / GE < qlen && 16 * w < rows_per_wg * GE;
+  if (kv_end > 0) load_tile(0);  // (a padded row has no keys at all)
+  for (int kv0 = 0; kv0 < kv_end; kv0 += BKV) {
+    __syncthreads();  // every wave is done reading the previous tile
+    store_tile();
+    __syncthreads();
+    if (kv0 + BKV < kv_end) load_tile(kv0 + BKV);
+    if (!wave_rows) continue;
+    if (kv0 > wave_qhi) continue;  // whole tile in this wave's causal future (barriers stay uniform)
+
+    f32x4 s[4];
+#pragma unroll
+    for (int kt = 0; kt < 4; ++kt) {
+      s[kt] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int ks = 0; ks < DK / 32; ++ks) {
+        const s16x8 kf = *reinterpret_cast<const s16x8*>(&Ks[(kt * 16 + li) * LDK + 32 * ks + 8 * g]);
+        s[kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[ks], s[kt], 0, 0, 0);
+      }
+    }
+    // S^T accumulators: lane (li, g) holds slot li's scores for keys kv0 + 16 kt + 4 g + i
+    float mx = m;
+#pragma unroll
+    for (int kt = 0; kt < 4; ++kt)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int key = kv0 + kt * 16 + 4 * g + i;
+        float v = s[kt][i] * scale;
+        if (cap > 0.f) {
+          const float e2 = __expf(2.0f * v * icap);  // tanh(x) = 1 - 2 / (exp(2x) + 1)
+          v = cap * (1.0f - 2.0f / (e2 + 1.0f));
+        }
+        v = (key <= qpos && key < kv_end) ? v : -1.0e30f;
+        s[kt][i] = v;
+        mx = fmaxf(mx, v);
+      }
+    mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    const float alpha = __expf(m - mx);
+    m = mx;
+    float ps = 0.f;
+    s16x8 pf[2];
+#pragma unroll
+    for (int kt = 0; kt < 4; ++kt)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float p = s[kt][i] > -1.0e29f ? __expf(s[kt][i] - mx) : 0.f;
+        const bf16_t pb = f2bf(p);
+        ps += bf2f(pb);
+        pf[kt >> 1][(kt & 1) * 4 + i] = (short)pb;
+      }
+    ps += __shfl_xor(ps, 16, 64);
+    ps += __shfl_xor(ps, 32, 64);
+    lsum = lsum * alpha + ps;
+#pragma unroll
+    for (int i = 0; i < NVT; ++i) o[i] *= alpha;
+
+    const int tq = li >> 2, tp = li & 3;
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks) {
+#pragma unroll
+      for (int dt = 0; dt < NVT; ++dt) {
+        const bf16_t* a0 = &Vs[(32 * ks + 4 * g + tq) * LDV + dt * 16 + 4 * tp];
+        const bf16_t* a1 = a0 + 16 * LDV;
+        const s16x4 x0 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LDS_AS s16x4*)(a0));
+        const s16x4 x1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LDS_AS s16x4*)(a1));
+        const s16x8 vf = {x0[0], x0[1], x0[2], x0[3], x1[0], x1[1], x1[2], x1[3]};
+        o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf[ks], o[dt], 0, 0, 0);
+      }
+    }
+  }
+  if (!valid) return;
+  const float inv = 1.0f / lsum;
+  float* op = out + ((int64_t)(t0 + row) * H + h) * RVtot + v0 + 4 * g;
+#pragma unroll
+  for (int dt = 0; dt < NVT; ++dt)
+    if (v0 + dt * 16 + 4 * g < RVtot) *reinterpret_cast<f32x4*>(op + dt * 16) = o[dt] * inv;
+}
+
+// Can the matrix-core kernel take this shape? (bf16 storage is the caller's to check.)
+bool sink_attn_mfma_ok(int dim, int vdim) { return (dim == 64 || dim == 128) && vdim % 8 == 0; }
+
+void launch_sink_attn_mfma(const void* q, const void* kc, const void* vc, const void* bt, int maxb, const void* cu,
+                           const void* ctx, void* out, int B, int max_qlen, int H, int G, int dim, int vdim, int bs,
+                           float scale, float cap, int all, hipStream_t st) {
+  if (B == 0 || max_qlen <= 0) return;
+  if (G < 1 || H % G) throw std::runtime_error("sink attention: heads must be a multiple of the key/value heads");
+  if (!sink_attn_mfma_ok(dim, vdim)) throw std::runtime_error("sink attention: shape not built for the matrix cores");
+  const int rep = H / G;
+  int GE = 1;
+  for (int ge = std::min(rep, 64); ge >= 1; --ge)
+    if (rep % ge == 0) {
+      GE = ge;
+      break;
+    }
+  const int rows_per_wg = 64 / GE;
+  const int RVtot = all ? G * vdim : vdim;
+  const int nvt = RVtot > 128 ? 16 : (RVtot > 64 ? 8 : 4);
+  const int nvch = (RVtot + nvt * 16 - 1) / (nvt * 16);
+  const int64_t gy = (int64_t)G * (rep / GE) * nvch;
+  if (gy > 65535 || B > 65535) throw std::runtime_error("sink attention: too many heads or sequences");
+  dim3 grid((max_qlen + rows_per_wg - 1) / rows_per_wg, (unsigned)gy, B);
+#define LAUNCH_SAM(DK_, NVT_)                                                                                       \
+  sink_attn_mfma_kernel<DK_, NVT_><<<grid, 256, 0, st>>>((const float*)q, (const bf16_t*)kc, (const bf16_t*)vc,      \
+                                                         (const int*)bt, maxb, (const int*)cu, (const int*)ctx,      \
+                                                         (float*)out, H, G, GE, vdim, bs, scale, cap, all, nvch)
+  if (dim == 64) {
+    if (nvt == 16) LAUNCH_SAM(64, 16);
+    else if (nvt == 8) LAUNCH_SAM(64, 8);
+    else LAUNCH_SAM(64, 4);
+  } else {
+    if (nvt == 16) LAUNCH_SAM(128, 16);
+    else if (nvt == 8) LAUNCH_SAM(128, 8);
+    else LAUNCH_SAM(128, 4);
+  }
+#undef LAUNCH_SAM
   HIP_CHECK_LAUNCH();
 }
 

@@ -8,15 +8,25 @@
 //                    beta = sigmoid(b), g = exp(-exp(A_log[head]) softplus(a + dt_bias[head]))
 //
 // Both updates act on the columns of S independently: column c needs only v[c] and the whole k and q. So a thread
-// owns one column (dim <= 128 values in registers; larger dims are split over 2 or 4 neighbouring lanes that
-// reduce with shuffles), and a workgroup owns (sequence, head, block of columns). Tokens are walked in order; the
-// rows of CT tokens at a time are staged in LDS by the whole workgroup (activation and the per-token scalars are
-// applied there). The state is read from the sequence's slot unless the portion starts at position 0 (then it is
+// owns one column, split over 1, 2 or 4 neighbouring lanes (32 to 128 state values in registers each) that reduce
+// with shuffles, and a workgroup owns (sequence, head, block of columns). Tokens are walked in order; the
+// rows of REC_CT tokens at a time are staged in LDS by the whole workgroup (activation and the per-token scalars
+// are applied there). The state is read from the sequence's slot unless the portion starts at position 0 (then it is
 // zero, whatever the slot held) and written back at the end. Rows of a padded sequence (no slot) are zeroed.
 #include "anytype.h"
 #include "seqrows.h"
 
-#define REC_CT 8
+#define REC_CT 8  // tokens staged at a time
+#define REC_NE 6  // staged numbers of a token per thread, at most: 5 of k / q / v and one per-token scalar
+
+// 32 consecutive floats from a 16-byte aligned LDS address
+__device__ __forceinline__ void ld32(const float* p, float* r) {
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const f32x4 v = *reinterpret_cast<const f32x4*>(p + 4 * i);
+    r[4 * i] = v[0], r[4 * i + 1] = v[1], r[4 * i + 2] = v[2], r[4 * i + 3] = v[3];
+  }
+}
 
 struct RecArgs {
   const void* q;  // [T, ldq]: head g's query at q + g * dim
@@ -37,18 +47,22 @@ struct RecArgs {
   int H, G, dim, vdim, silu_in;
 };
 
-// TQ: storage of q / k / v; TP: storage of a / b. R: state values per lane, P lanes per column.
+// TQ: storage of q / k / v; TP: storage of a / b. R: state values per lane, P lanes per column. Staging: every
+// thread owns up to REC_NE of a token's `per` staged numbers (k [dim], q [dim], v [cols], beta, g); the next REC_CT
+// tokens' numbers are fetched into registers before the current ones are computed on, and put into LDS afterwards,
+// so the global loads are in flight behind the arithmetic. Threads beyond cols * P only fetch.
 template <typename TQ, typename TP, int R, int MODE>
 __global__ __launch_bounds__(256) void recurrence_kernel(RecArgs A, int P, int cols) {
-  extern __shared__ float sm[];
+  extern __shared__ __attribute__((aligned(16))) float sm[];
   const int b = blockIdx.x, h = blockIdx.y;
   const int dim = A.dim, vdim = A.vdim;
   const int g = h / (A.H / A.G);
   const int qlen = A.cu[b + 1] - A.cu[b];
   if (qlen <= 0) return;
   const int t0 = A.cu[b], n = A.ctx[b], slot = A.sslots[b];
-  const int col = blockIdx.z * cols + threadIdx.x / P, part = threadIdx.x % P;
-  const bool live = col < vdim && threadIdx.x / P < cols;
+  const int cidx = min((int)threadIdx.x / P, cols - 1);
+  const int col = blockIdx.z * cols + cidx, part = threadIdx.x % P;
+  const bool live = col < vdim && (int)threadIdx.x < cols * P;
   if (slot < 0 || n <= 0) {
     if (live && part == 0)
       for (int j = 0; j < qlen; ++j) A.out[(int64_t)(t0 + j) * A.ldo + (int64_t)h * vdim + col] = 0.f;
@@ -58,10 +72,19 @@ __global__ __launch_bounds__(256) void recurrence_kernel(RecArgs A, int P, int c
   const int d0 = part * R;  // this lane's rows of the column: d0 .. d0 + R - 1
   float S[R];
   float* sp = A.state + (((int64_t)slot * A.H + h) * dim) * vdim;
+  if (p0 > 0) {  // rows past dim and lanes without a column read a valid address and drop the value
+    const int cc = min(col, vdim - 1);
 #pragma unroll
-  for (int i = 0; i < R; ++i) S[i] = (live && p0 > 0 && d0 + i < dim) ? sp[(int64_t)(d0 + i) * vdim + col] : 0.f;
-  // LDS per staged token: k [dim], q [dim], v [cols], 2 scalars
-  const int per = 2 * dim + cols + 2;
+    for (int i = 0; i < R; ++i) S[i] = sp[(int64_t)min(d0 + i, dim - 1) * vdim + cc];
+#pragma unroll
+    for (int i = 0; i < R; ++i) S[i] = (live && d0 + i < dim) ? S[i] : 0.f;
+  } else {
+#pragma unroll
+    for (int i = 0; i < R; ++i) S[i] = 0.f;
+  }
+  // staged numbers per token: k [dimp], q [dimp], v [cols], beta, g; rows padded to whole 16-byte reads
+  const int dimp = (dim + 3) & ~3;
+  const int per = (2 * dimp + cols + 2 + 3) & ~3;
   float a_const = 0.f, dtb = 0.f;
   if (MODE == 0) a_const = A.decay[h];
   else {
@@ -69,82 +92,135 @@ __global__ __launch_bounds__(256) void recurrence_kernel(RecArgs A, int P, int c
     dtb = A.dt_bias[h];
   }
   const float qmul = MODE == 1 ? 1.0f / sqrtf((float)dim) : 1.0f;
+  // this thread's staged numbers: slots 0 .. REC_NE - 2 hold k / q / v entries (storage TQ), the last slot the
+  // head's two per-token scalars (storage TP, threads 0 and 1). A slot without an entry points at a valid address
+  // all the same, so every load is unconditional and the whole batch is in flight together.
+  const TQ* src[REC_NE - 1];
+  int64_t ld[REC_NE - 1];
+  bool has[REC_NE - 1];
+  const TQ* dummy = (const TQ*)A.k + (int64_t)t0 * A.ldk + (int64_t)g * dim;
+#pragma unroll
+  for (int k = 0; k < REC_NE - 1; ++k) {
+    const int e = threadIdx.x + k * blockDim.x;
+    has[k] = false, src[k] = dummy, ld[k] = A.ldk;
+    if (e < dimp) {
+      if (e < dim) has[k] = true, src[k] = dummy + e;
+    } else if (e < 2 * dimp) {
+      if (e - dimp < dim)
+        has[k] = true, ld[k] = A.ldq, src[k] = (const TQ*)A.q + (int64_t)t0 * A.ldq + (int64_t)g * dim + (e - dimp);
+    } else if (e < 2 * dimp + cols) {
+      const int c = blockIdx.z * cols + (e - 2 * dimp);
+      if (c < vdim) has[k] = true, ld[k] = A.ldv, src[k] = (const TQ*)A.v + (int64_t)t0 * A.ldv + (int64_t)h * vdim + c;
+    }
+  }
+  const bool has_s = MODE == 1 && threadIdx.x < 2;  // thread 0: beta's input, thread 1: the decay's
+  const TP* src_s = has_s ? (const TP*)A.ab + (int64_t)t0 * A.ldab + (threadIdx.x == 0 ? A.off_b : A.off_a) + h : nullptr;
+  float pre[REC_CT * REC_NE];
+  auto fetch = [&](int j0) {
+#pragma unroll
+    for (int jj = 0; jj < REC_CT; ++jj) {
+      const int64_t tj = min(j0 + jj, qlen - 1);
+#pragma unroll
+      for (int k = 0; k < REC_NE - 1; ++k) pre[jj * REC_NE + k] = El<TQ>::ld(src[k] + tj * ld[k]);
+      if (MODE == 1) pre[jj * REC_NE + REC_NE - 1] = has_s ? El<TP>::ld(src_s + tj * A.ldab) : 0.f;
+    }
+  };
+  auto put = [&]() {
+#pragma unroll
+    for (int jj = 0; jj < REC_CT; ++jj) {
+#pragma unroll
+      for (int k = 0; k < REC_NE - 1; ++k) {
+        const int e = threadIdx.x + k * blockDim.x;
+        if (e >= 2 * dimp + cols) continue;
+        float v = has[k] ? pre[jj * REC_NE + k] : 0.f;
+        if (A.silu_in) v = v / (1.0f + expf(-v));
+        sm[jj * per + e] = v;
+      }
+      if (has_s) {
+        float v = pre[jj * REC_NE + REC_NE - 1];
+        if (threadIdx.x == 0) {
+          v = 1.0f / (1.0f + expf(-v));
+        } else {
+          const float z = v + dtb;
+          v = expf(-a_const * (z > 20.f ? z : log1pf(expf(z))));
+        }
+        sm[jj * per + 2 * dimp + cols + threadIdx.x] = v;
+      }
+    }
+  };
+  fetch(0);
   for (int j0 = 0; j0 < qlen; j0 += REC_CT) {
     const int nt = min(REC_CT, qlen - j0);
+    __syncthreads();  // the previous tokens' readers are done
+    put();
     __syncthreads();
-    for (int idx = threadIdx.x; idx < nt * per; idx += blockDim.x) {
-      const int jj = idx / per, e = idx % per;
-      const int64_t t = t0 + j0 + jj;
-      float val;
-      if (e < 2 * dim) {
-        const bool isq = e >= dim;
-        const int d = isq ? e - dim : e;
-        const TQ* src = isq ? (const TQ*)A.q + t * A.ldq : (const TQ*)A.k + t * A.ldk;
-        val = El<TQ>::ld(src + (int64_t)g * dim + d);
-        if (A.silu_in) val = val / (1.0f + expf(-val));
-      } else if (e < 2 * dim + cols) {
-        const int c = blockIdx.z * cols + (e - 2 * dim);
-        val = c < vdim ? El<TQ>::ld((const TQ*)A.v + t * A.ldv + (int64_t)h * vdim + c) : 0.f;
-        if (A.silu_in) val = val / (1.0f + expf(-val));
-      } else if (MODE == 1) {
-        const TP* ab = (const TP*)A.ab + t * A.ldab;
-        if (e == 2 * dim + cols) {  // beta
-          val = 1.0f / (1.0f + expf(-El<TP>::ld(ab + A.off_b + h)));
-        } else {  // g
-          const float z = El<TP>::ld(ab + A.off_a + h) + dtb;
-          const float sp_ = z > 20.f ? z : log1pf(expf(z));
-          val = expf(-a_const * sp_);
-        }
-      } else {
-        val = 0.f;
-      }
-      sm[idx] = val;
-    }
-    __syncthreads();
+    if (j0 + REC_CT < qlen) fetch(j0 + REC_CT);
     for (int jj = 0; jj < nt; ++jj) {
       const float* ks = sm + jj * per;
-      const float* qs = ks + dim;
-      const float vv = ks[2 * dim + min((int)threadIdx.x / P, cols - 1)];
-      float o = 0.f;
+      const float* qs = ks + dimp;
+      const float vv = ks[2 * dimp + cidx];
+      // k and q come from LDS 32 numbers at a time by 16-byte reads issued together (a wave alone on its SIMD has
+      // nobody to hide a read's latency behind), sums run in four partial accumulators
+      float o4[4] = {0.f, 0.f, 0.f, 0.f};
       if (MODE == 0) {
 #pragma unroll
-        for (int i = 0; i < R; ++i) {
-          if (d0 + i < dim) {
-            S[i] = fmaf(a_const, S[i], ks[d0 + i] * vv);
-            o = fmaf(S[i], qs[d0 + i], o);
-          }
-        }
-        for (int m = 1; m < P; m <<= 1) o += __shfl_xor(o, m, 64);
-      } else {
-        const float beta = ks[2 * dim + cols], gg = ks[2 * dim + cols + 1];
-        float kk = 0.f, qq = 0.f, sk = 0.f;
+        for (int c0 = 0; c0 < R; c0 += 32) {
+          float kr[32], qr[32];
+          ld32(ks + d0 + c0, kr);
+          ld32(qs + d0 + c0, qr);
 #pragma unroll
-        for (int i = 0; i < R; ++i) {
-          if (d0 + i < dim) {
-            const float kd = ks[d0 + i], qd = qs[d0 + i];
-            kk = fmaf(kd, kd, kk);
-            qq = fmaf(qd, qd, qq);
-            S[i] *= gg;
-            sk = fmaf(S[i], kd, sk);
+          for (int i = 0; i < 32; ++i) {
+            if (d0 + c0 + i < dim) {
+              S[c0 + i] = fmaf(a_const, S[c0 + i], kr[i] * vv);
+              o4[i & 3] = fmaf(S[c0 + i], qr[i], o4[i & 3]);
+            }
           }
         }
+      } else {
+        const float beta = ks[2 * dimp + cols], gg = ks[2 * dimp + cols + 1];
+        float kk4[4] = {0.f, 0.f, 0.f, 0.f}, sk4[4] = {0.f, 0.f, 0.f, 0.f}, qq4[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int c0 = 0; c0 < R; c0 += 32) {
+          float kr[32];
+          ld32(ks + d0 + c0, kr);
+#pragma unroll
+          for (int i = 0; i < 32; ++i) {
+            if (d0 + c0 + i < dim) {
+              kk4[i & 3] = fmaf(kr[i], kr[i], kk4[i & 3]);
+              S[c0 + i] *= gg;
+              sk4[i & 3] = fmaf(S[c0 + i], kr[i], sk4[i & 3]);
+            }
+          }
+        }
+        float kk = (kk4[0] + kk4[1]) + (kk4[2] + kk4[3]), sk = (sk4[0] + sk4[1]) + (sk4[2] + sk4[3]);
         for (int m = 1; m < P; m <<= 1) {
           kk += __shfl_xor(kk, m, 64);
-          qq += __shfl_xor(qq, m, 64);
           sk += __shfl_xor(sk, m, 64);
         }
-        const float kn = 1.0f / sqrtf(kk + 1e-6f), qn = qmul / sqrtf(qq + 1e-6f);
-        const float u = beta * (vv - sk * kn);
+        const float kn = 1.0f / sqrtf(kk + 1e-6f);
+        const float u = beta * (vv - sk * kn) * kn;
 #pragma unroll
-        for (int i = 0; i < R; ++i) {
-          if (d0 + i < dim) {
-            S[i] = fmaf(ks[d0 + i] * kn, u, S[i]);
-            o = fmaf(S[i], qs[d0 + i], o);
+        for (int c0 = 0; c0 < R; c0 += 32) {
+          float kr[32], qr[32];
+          ld32(ks + d0 + c0, kr);
+          ld32(qs + d0 + c0, qr);
+#pragma unroll
+          for (int i = 0; i < 32; ++i) {
+            if (d0 + c0 + i < dim) {
+              qq4[i & 3] = fmaf(qr[i], qr[i], qq4[i & 3]);
+              S[c0 + i] = fmaf(kr[i], u, S[c0 + i]);
+              o4[i & 3] = fmaf(S[c0 + i], qr[i], o4[i & 3]);
+            }
           }
         }
-        for (int m = 1; m < P; m <<= 1) o += __shfl_xor(o, m, 64);
-        o *= qn;
+        float qq = (qq4[0] + qq4[1]) + (qq4[2] + qq4[3]);
+        for (int m = 1; m < P; m <<= 1) qq += __shfl_xor(qq, m, 64);
+        const float qn = qmul / sqrtf(qq + 1e-6f);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) o4[i] *= qn;
       }
+      float o = (o4[0] + o4[1]) + (o4[2] + o4[3]);
+      for (int m = 1; m < P; m <<= 1) o += __shfl_xor(o, m, 64);
       if (live && part == 0) A.out[(int64_t)(t0 + j0 + jj) * A.ldo + (int64_t)h * vdim + col] = o;
     }
   }
@@ -155,19 +231,23 @@ __global__ __launch_bounds__(256) void recurrence_kernel(RecArgs A, int P, int c
   }
 }
 
+// A column is split over up to 4 lanes (32 state values per lane up to dim 128): more waves share the walk, and the
+// state, the staged k / q and the prefetched rows fit the register file without spilling.
 template <typename TQ, typename TP, int MODE>
 static void recurrence_t(const RecArgs& A, int B, hipStream_t st) {
   const int dim = A.dim, vdim = A.vdim;
   int P = 1;
-  while (P < 4 && dim > 128 * P) P <<= 1;
+  while (P < 4 && dim > 32 * P) P <<= 1;
   if (dim > 128 * P) throw std::runtime_error("recurrence: key dimension above 512");
-  const int per_lane = (dim + P - 1) / P;
-  const int R = per_lane <= 32 ? 32 : (per_lane <= 64 ? 64 : 128);
-  const int cols = std::min(vdim, 64 / P);  // one wave per workgroup: many small workgroups fill the chip
-  const int threads = ((cols * P + 63) / 64) * 64;
+  const int R = dim <= 32 * P ? 32 : (dim <= 64 * P ? 64 : 128);
+  const int cols = std::min(vdim, 64 / P);  // a wave of state columns per workgroup: many workgroups fill the chip
+  const int dimp = (dim + 3) & ~3;
+  const int per = (2 * dimp + cols + 2 + 3) & ~3;
+  const int threads = ((std::max(cols * P, (2 * dimp + cols + REC_NE - 2) / (REC_NE - 1)) + 63) / 64) * 64;
+  if (threads > 256) throw std::runtime_error("recurrence: too many numbers per token to stage");
   dim3 g(B, A.H, (vdim + cols - 1) / cols);
   if (A.H > 65535 || g.z > 65535) throw std::runtime_error("recurrence: too many heads or columns");
-  const size_t lds = (size_t)REC_CT * (2 * dim + cols + 2) * 4;
+  const size_t lds = ((size_t)REC_CT * per + 4 * 128) * 4;  // + room for the last token's reads past its k / q
   if (R == 32) recurrence_kernel<TQ, TP, 32, MODE><<<g, threads, lds, st>>>(A, P, cols);
   else if (R == 64) recurrence_kernel<TQ, TP, 64, MODE><<<g, threads, lds, st>>>(A, P, cols);
   else recurrence_kernel<TQ, TP, 128, MODE><<<g, threads, lds, st>>>(A, P, cols);

@@ -131,8 +131,10 @@ class ParallelMixer:
         q = ops.rope_bias_cache(proj, c["lq"], c["lk"], c["lv"], W.bias, inp.positions, W.angles,
                                 a.rot.dims if a.rot is not None else 0, kc, vc, inp.slots, a.heads, a.kv_heads, a.dim,
                                 a.vdim)
+        single = inp.kind == "decode"
         O = ops.sink_attn(q, kc, vc, inp.block_tables, cu, inp.ctx_lens, a.heads, a.kv_heads, a.dim, a.vdim, a.scale,
-                          a.softcap, W.talk is not None)
+                          a.softcap, W.talk is not None, max_qlen=1 if single else max(1, inp.max_seqlen),
+                          num_decode=0 if single else inp.num_decode)
         nl, nr = a.heads * a.vdim, r.heads * r.vdim
         both = torch.empty(T, nl + nr, dtype=dt, device=h.device)  # [left | right] rows for the one output GEMM
         ops.talk_mix(O, W.talk, spec.left_scale, a.heads, a.kv_heads, a.vdim, out=both[:, :nl])

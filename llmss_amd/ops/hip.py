@@ -1257,7 +1257,10 @@ def rope_bias_cache(proj, off_q, off_k, off_v, bias, positions, table, rot, k_ca
 
 
 def sink_attn(q, k_cache, v_cache, block_tables, cu, ctx_lens, heads, kv_heads, dim, vdim, scale, softcap,
-              all_groups):
+              all_groups, max_qlen=0, num_decode=0):
+    """``max_qlen`` (the longest portion of the step, known on the host) > 0: a bf16 cache of a shape the matrix-core
+    kernel is built for runs on it, portions and single rows alike (``num_decode`` leading single-row sequences are
+    part of its grid); everything else runs the vector kernel."""
     T = q.shape[0]
     _rows(q, "q", heads * dim, torch.float32)
     _check(q.is_contiguous(), "q contiguous")
@@ -1271,10 +1274,19 @@ def sink_attn(q, k_cache, v_cache, block_tables, cu, ctx_lens, heads, kv_heads, 
            and k_cache.shape[:2] == v_cache.shape[:2], "k / v cache [blocks, block_size, kv_heads * dim | vdim]")
     R = kv_heads * vdim if all_groups else vdim
     out = torch.empty(T, heads, R, dtype=torch.float32, device=q.device)
-    lib().sink_attn(q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), block_tables.data_ptr(),
-                    block_tables.shape[1], cu.data_ptr(), ctx_lens.data_ptr(), out.data_ptr(), T, B, heads, kv_heads,
-                    dim, vdim, k_cache.shape[1], float(scale), float(softcap or 0.0), int(bool(all_groups)),
-                    _dt(k_cache, "k cache"), _stream())
+    nd = int(num_decode)
+    _check(0 <= nd <= B, "num_decode outside the step")
+    mfma = (k_cache.dtype == torch.bfloat16 and max_qlen > 0 and lib().sink_attn_mfma_ok(dim, vdim)
+            and k_cache.data_ptr() % 16 == 0 and v_cache.data_ptr() % 16 == 0 and os.environ.get("LLMSS_SINK_MFMA", "1") != "0")
+    common = (heads, kv_heads, dim, vdim, k_cache.shape[1], float(scale), float(softcap or 0.0), int(bool(all_groups)))
+    if mfma:
+        lib().sink_attn_mfma(q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), block_tables.data_ptr(),
+                             block_tables.shape[1], cu.data_ptr(), ctx_lens.data_ptr(), out.data_ptr(), B,
+                             int(max_qlen), *common, _stream())
+    else:
+        lib().sink_attn(q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), block_tables.data_ptr(),
+                        block_tables.shape[1], cu.data_ptr(), ctx_lens.data_ptr(), out.data_ptr(), T, B, *common,
+                        _dt(k_cache, "k cache"), _stream())
     return out
 
 

@@ -761,11 +761,12 @@ def rope_bias_cache(proj, off_q: int, off_k: int, off_v: int, bias, positions, t
 
 
 def sink_attn(q, k_cache, v_cache, block_tables, cu, ctx_lens, heads: int, kv_heads: int, dim: int, vdim: int,
-              scale: float, softcap: float, all_groups: bool):
+              scale: float, softcap: float, all_groups: bool, max_qlen: int = 0, num_decode: int = 0):
     """Causal attention of every row over its sequence's cached keys with a sink in the softmax denominator
     (p_j = exp(s_j) / (1 + sum exp(s))) and optionally soft-capped scores. Returns fp32 [T, heads, R]: head h's
     weights applied to the value rows of every group side by side (``all_groups``, R = kv_heads * vdim) or of its
-    own group only (R = vdim)."""
+    own group only (R = vdim). ``max_qlen`` (longest portion) and ``num_decode`` (leading single-row sequences) only
+    steer the choice of GPU kernel."""
     T = q.shape[0]
     bs = k_cache.shape[1]
     rep = heads // kv_heads

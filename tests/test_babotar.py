@@ -68,6 +68,18 @@ CONFIGS = {
         lig(2, 160, 72, [0.9, 0.999], ff=64),
     ]),
 }
+CONFIGS.update({
+    # odd sizes everywhere (no dimension a multiple of 8), five streams, a rotation of two dimensions
+    "odd": dict(architecture="Babotar", vocab=51, width=36, max_positions=160, norm=dict(eps=1e-5),
+                residual_mult=0.9, streams=5, canon=dict(taps=2), layers=[
+        par(left(6, 3, 6, 5, 0.4, softcap=8.0, rot=dict(base=50.0, dims=2, scaling=YARN)),
+            dict(heads=3, kv_heads=3, dim=5, vdim=7, conv=3), 1.0, 1.0, ff=27),
+        lig(5, 3, 9, [0.5, 0.7, 0.9, 0.95, 0.99], ff=19),
+    ]),
+    # no attention at all: nothing is paged, everything a sequence keeps lives in its state slot
+    "decays": dict(architecture="Babotar", vocab=43, width=32, max_positions=160, norm=dict(eps=1e-5),
+                   streams=2, layers=[lig(2, 8, 8, [0.7, 0.97], ff=40), lig(4, 4, 12, [0.5, 0.8, 0.9, 0.999])]),
+})
 DROP = {"plain": (".talk", ".q.b", ".k.b", ".v.b")}  # checkpoints without head mixing and without biases
 
 

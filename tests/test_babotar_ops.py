@@ -62,7 +62,7 @@ def meta(step, slots, device):
 def test_stream_write_back_and_normed_read(device, dtype, S, W, rms):
     T = 7
     x0 = rnd(S, T, W, seed=1) * 3 + 0.5
-    y, w = rnd(T, W, seed=2, dtype=dtype), 1 + 0.1 * rnd(W, seed=3, dtype=dtype)
+    y, w = rnd(T, W, seed=2, dtype=dtype), (1 + 0.1 * rnd(W, seed=3)).to(dtype).double()
     mix, outw, inw = torch.eye(S).double() + 0.3 * rnd(S, S, seed=4), 1 + 0.3 * rnd(S, seed=5), rnd(S, seed=6)
     c, eps = 0.7, 1e-5
     x = x0.float().to(device).contiguous()
@@ -278,6 +278,8 @@ def attention_case(device, dtype, H, G, d, dv, lens, cuts, scale, cap, talk, bs=
     tk = (torch.eye(H).double() * 0.5 + 0.4 * rnd(H, H, seed=9)) if talk else None
     got = [torch.zeros(n, H * dv) for n in lens]
     for step in steps_of(cuts):
+        step = sorted(step, key=lambda e: not (e[2] == 1 and e[1] > 0))  # single rows after a prefix come first
+        nd = sum(1 for _, p0, n in step if n == 1 and p0 > 0)
         seqs = [s for s, _, _ in step]
         for s, p0, n in step:  # the step's keys and values are in the cache before it attends
             sl = torch.tensor(pg.slots(s, p0, n), device=device)
@@ -285,7 +287,8 @@ def attention_case(device, dtype, H, G, d, dv, lens, cuts, scale, cap, talk, bs=
             pg.vc.view(-1, G * dv)[sl] = data[s][2][p0:p0 + n].reshape(n, -1).to(dtype).to(device)
         cu, ctx, _ = meta(step, [0] * len(lens), device)
         q = torch.cat([data[s][0][p0:p0 + n] for s, p0, n in step]).reshape(-1, H * d).float().to(device)
-        O = ops.sink_attn(q, pg.kc, pg.vc, pg.bt(seqs, device), cu, ctx, H, G, d, dv, scale, cap, talk)
+        O = ops.sink_attn(q, pg.kc, pg.vc, pg.bt(seqs, device), cu, ctx, H, G, d, dv, scale, cap, talk,
+                          max_qlen=max(n for _, _, n in step), num_decode=nd)
         y = ops.talk_mix(O, tk.float().to(device).contiguous() if talk else None, 0.8, H, G, dv,
                          out_dtype=torch.float32).cpu()
         r = 0
@@ -301,17 +304,22 @@ def attention_case(device, dtype, H, G, d, dv, lens, cuts, scale, cap, talk, bs=
 
 @pytest.mark.parametrize("device,dtype", RUNS)
 @pytest.mark.parametrize("H,G,d,dv,talk", [(4, 2, 16, 12, True), (4, 4, 8, 20, True), (3, 1, 24, 40, False),
-                                           (1, 1, 8, 8, True), (8, 2, 64, 72, True), (16, 2, 32, 8, False)])
+                                           (1, 1, 8, 8, True), (8, 2, 64, 72, True), (16, 2, 32, 8, False),
+                                           (4, 2, 128, 64, True), (4, 1, 128, 40, False), (6, 2, 64, 160, True),
+                                           (2, 2, 64, 128, False)])
 def test_sink_attention_portions_decoding_and_batches(device, dtype, H, G, d, dv, talk):
+    # key sizes 64 and 128 with value sizes in eights: in bf16 on a GPU the portions run on the matrix cores
     attention_case(device, dtype, H, G, d, dv, [70, 1, 33], [[16, 1, 15, 2, 1, 1, 30, 3, 1], [1], [2, 31]],
                    d ** -0.5, 30.0, talk)
+    attention_case(device, dtype, H, G, d, dv, [150, 90], [[65, 64, 1, 20], [3, 87]], d ** -0.5, 0.0, talk, seed=7)
 
 
 @pytest.mark.parametrize("device,dtype", RUNS)
+@pytest.mark.parametrize("d", [16, 64])
 @pytest.mark.parametrize("far", [0, 15, 16, 17, 63, 64, 200])
-def test_a_far_key_among_hundreds_in_a_prompt_and_when_decoding(device, dtype, far):
+def test_a_far_key_among_hundreds_in_a_prompt_and_when_decoding(device, dtype, far, d):
     # the last query of the prompt portion and the decoded token both point at one key far back / at a page border
-    H, G, d, dv, n = 2, 1, 16, 8, 300
+    H, G, dv, n = 2, 1, 8, 300
     got, data = attention_case(device, dtype, H, G, d, dv, [n], [[n - 1, 1]], 0.25, 0.0, False, boost=(0, far, 6.0),
                                seed=100 + far)
     q, k, v = data[0]
