@@ -18,6 +18,10 @@ Families (``MODEL_REGISTRY`` keys, reference ``custom_modeling/__init__.py:4-7``
 * ``timisun``     - per-layer description (``layer_specs``): parallel blocks over an fp32 residual, latent
                     attention without positions (sliding window, latent rows shared between layers),
                     mixture-of-experts feed-forward with a shared expert, scaled embedding, tied head.
+* ``babotar``     - per-layer description: sequential pre-norm blocks (bias-free layer norm) over one or several
+                    fp32 residual streams, optional causal input convolution, mixers ``parallel`` (sink attention
+                    beside a gated delta rule) and ``lightning`` (decay linear attention), gated tanh-GELU
+                    feed-forward, learned positions, untied head.
 """
 from __future__ import annotations
 
