@@ -28,6 +28,20 @@ __device__ __forceinline__ void ld32(const float* p, float* r) {
   }
 }
 
+// Sum over the 1, 2 or 4 neighbouring lanes that share a state column: lane-swap moves inside a quad (data-parallel
+// primitives on the vector ALU; no trip through LDS as a general shuffle would take)
+__device__ __forceinline__ float quad_swap1(float v) {  // lanes 0 <-> 1, 2 <-> 3
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0xB1, 0xF, 0xF, false));
+}
+__device__ __forceinline__ float quad_swap2(float v) {  // lanes 0 <-> 2, 1 <-> 3
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x4E, 0xF, 0xF, false));
+}
+__device__ __forceinline__ float part_sum(float v, int P) {
+  if (P >= 2) v += quad_swap1(v);
+  if (P >= 4) v += quad_swap2(v);
+  return v;
+}
+
 struct RecArgs {
   const void* q;  // [T, ldq]: head g's query at q + g * dim
   const void* k;
@@ -133,7 +147,7 @@ __global__ __launch_bounds__(256) void recurrence_kernel(RecArgs A, int P, int c
         const int e = threadIdx.x + k * blockDim.x;
         if (e >= 2 * dimp + cols) continue;
         float v = has[k] ? pre[jj * REC_NE + k] : 0.f;
-        if (A.silu_in) v = v / (1.0f + expf(-v));
+        if (A.silu_in) v = v / (1.0f + (sizeof(TQ) == 2 ? __expf(-v) : expf(-v)));  // bf16 rows: the fast exponential
         sm[jj * per + e] = v;
       }
       if (has_s) {
@@ -193,10 +207,8 @@ __global__ __launch_bounds__(256) void recurrence_kernel(RecArgs A, int P, int c
           }
         }
         float kk = (kk4[0] + kk4[1]) + (kk4[2] + kk4[3]), sk = (sk4[0] + sk4[1]) + (sk4[2] + sk4[3]);
-        for (int m = 1; m < P; m <<= 1) {
-          kk += __shfl_xor(kk, m, 64);
-          sk += __shfl_xor(sk, m, 64);
-        }
+        kk = part_sum(kk, P);
+        sk = part_sum(sk, P);
         const float kn = 1.0f / sqrtf(kk + 1e-6f);
         const float u = beta * (vv - sk * kn) * kn;
 #pragma unroll
@@ -214,13 +226,13 @@ __global__ __launch_bounds__(256) void recurrence_kernel(RecArgs A, int P, int c
           }
         }
         float qq = (qq4[0] + qq4[1]) + (qq4[2] + qq4[3]);
-        for (int m = 1; m < P; m <<= 1) qq += __shfl_xor(qq, m, 64);
+        qq = part_sum(qq, P);
         const float qn = qmul / sqrtf(qq + 1e-6f);
 #pragma unroll
         for (int i = 0; i < 4; ++i) o4[i] *= qn;
       }
       float o = (o4[0] + o4[1]) + (o4[2] + o4[3]);
-      for (int m = 1; m < P; m <<= 1) o += __shfl_xor(o, m, 64);
+      o = part_sum(o, P);
       if (live && part == 0) A.out[(int64_t)(t0 + j0 + jj) * A.ldo + (int64_t)h * vdim + col] = o;
     }
   }

@@ -15,6 +15,7 @@
 
 #define MAX_STREAMS 8
 #define MAX_TAIL 8
+#define CONV_CPT 4  // channels per thread of the convolution kernel
 
 // x[s, t, :] = table[ids[t], :] (+ pos_table[positions[t], :]) for every stream s
 template <typename T>
@@ -134,26 +135,29 @@ __global__ __launch_bounds__(256) void causal_conv_kernel(const TI* __restrict__
                                                           const int* __restrict__ cu, const int* __restrict__ ctx,
                                                           const int* __restrict__ sslots, TO* __restrict__ out,
                                                           int64_t ldo, int B, int C, int taps, int res, int silu) {
-  const int t = blockIdx.x, c = blockIdx.y * blockDim.x + threadIdx.x;
-  if (c >= C) return;
-  const RowSeq r = row_seq(cu, ctx, B, t);
+  const int t = blockIdx.x;
+  const RowSeq r = row_seq(cu, ctx, B, t);  // once per workgroup: a thread walks CONV_CPT channels
+  const int c_end = min(C, (int)(blockIdx.y + 1) * (int)blockDim.x * CONV_CPT);
   if (r.pos < 0) {
-    El<TO>::st(out + (int64_t)t * ldo + c, 0.f);
+    for (int c = blockIdx.y * blockDim.x * CONV_CPT + threadIdx.x; c < c_end; c += blockDim.x)
+      El<TO>::st(out + (int64_t)t * ldo + c, 0.f);
     return;
   }
   const int slot = sslots[r.b];
   const int R = taps - 1;
-  float acc = res ? El<TI>::ld(in + (int64_t)t * ldi + c) : 0.f;
-  for (int k = 0; k < taps; ++k) {
-    const int d = R - k;
-    if (r.pos - d < 0) continue;
-    float v;
-    if (r.j - d >= 0) v = El<TI>::ld(in + (int64_t)(t - d) * ldi + c);
-    else v = state[((int64_t)slot * R + (r.j - d + R)) * C + c];
-    acc = fmaf(El<TW>::ld(w + (int64_t)c * taps + k), v, acc);
+  for (int c = blockIdx.y * blockDim.x * CONV_CPT + threadIdx.x; c < c_end; c += blockDim.x) {
+    float acc = res ? El<TI>::ld(in + (int64_t)t * ldi + c) : 0.f;
+    for (int k = 0; k < taps; ++k) {
+      const int d = R - k;
+      if (r.pos - d < 0) continue;
+      float v;
+      if (r.j - d >= 0) v = El<TI>::ld(in + (int64_t)(t - d) * ldi + c);
+      else v = state[((int64_t)slot * R + (r.j - d + R)) * C + c];
+      acc = fmaf(El<TW>::ld(w + (int64_t)c * taps + k), v, acc);
+    }
+    if (silu) acc = acc / (1.0f + expf(-acc));
+    El<TO>::st(out + (int64_t)t * ldo + c, acc);
   }
-  if (silu) acc = acc / (1.0f + expf(-acc));
-  El<TO>::st(out + (int64_t)t * ldo + c, acc);
 }
 
 // The tail after the step: state[slot, i, c] <- input at position ctx - (taps - 1) + i
@@ -187,7 +191,7 @@ template <typename TI, typename TW, typename TO>
 static void causal_conv_t(const void* in, int64_t ldi, const void* w, void* state, const void* cu, const void* ctx,
                           const void* sslots, void* out, int64_t ldo, int T_, int B, int C, int taps, int res,
                           int silu, hipStream_t st) {
-  dim3 g(T_, (C + 255) / 256);
+  dim3 g(T_, (C + 256 * CONV_CPT - 1) / (256 * CONV_CPT));
   causal_conv_kernel<TI, TW, TO><<<g, 256, 0, st>>>((const TI*)in, ldi, (const TW*)w, (const float*)state,
                                                     (const int*)cu, (const int*)ctx, (const int*)sslots, (TO*)out, ldo,
                                                     B, C, taps, res, silu);
