@@ -127,7 +127,10 @@ void launch_glu_act(const void* gu, int64_t ldg, void* out, int64_t ldo, int T_,
 void launch_recurrence(int mode, const void* q, const void* k, const void* v, int64_t ldq, int64_t ldk, int64_t ldv,
                        const void* ab, int64_t ldab, int off_a, int off_b, const void* decay, const void* dt_bias,
                        void* state, const void* cu, const void* ctx, const void* sslots, void* out, int64_t ldo, int B,
-                       int H, int G, int dim, int vdim, int silu_in, int dq, int dp, hipStream_t st);
+                       int H, int G, int dim, int vdim, int silu_in, int gates_ready, int dq, int dp, hipStream_t st);
+void launch_silu_f32(const void* in, int64_t ldi, void* out, int64_t ldo, int T_, int n, int dt, hipStream_t st);
+void launch_delta_gates(const void* a, const void* b, int64_t ld, const void* A_log, const void* dt_bias, void* gates,
+                        int T_, int H, int dt, hipStream_t st);
 void launch_rope_bias_cache(const void* proj, int64_t ldp, int off_q, int off_k, int off_v, const void* bias,
                             const void* positions, const void* cs, int npos, int rot, void* qout, void* kc, void* vc,
                             const void* slots, int T_, int H, int G, int dim, int vdim, int dt, hipStream_t st);
@@ -364,9 +367,16 @@ PYBIND11_MODULE(_C, m) {
   m.def("recurrence", [](int mode, uintptr_t q, uintptr_t k, uintptr_t v, int64_t ldq, int64_t ldk, int64_t ldv,
                          uintptr_t ab, int64_t ldab, int off_a, int off_b, uintptr_t decay, uintptr_t dtb,
                          uintptr_t state, uintptr_t cu, uintptr_t ctx, uintptr_t ss, uintptr_t out, int64_t ldo, int B,
-                         int H, int G, int dim, int vdim, int silu_in, int dq, int dp, uintptr_t st) {
+                         int H, int G, int dim, int vdim, int silu_in, int gates_ready, int dq, int dp, uintptr_t st) {
     launch_recurrence(mode, CP(q), CP(k), CP(v), ldq, ldk, ldv, CP(ab), ldab, off_a, off_b, CP(decay), CP(dtb),
-                      P(state), CP(cu), CP(ctx), CP(ss), P(out), ldo, B, H, G, dim, vdim, silu_in, dq, dp, S(st));
+                      P(state), CP(cu), CP(ctx), CP(ss), P(out), ldo, B, H, G, dim, vdim, silu_in, gates_ready, dq, dp, S(st));
+  });
+  m.def("silu_f32", [](uintptr_t in, int64_t ldi, uintptr_t out, int64_t ldo, int T, int n, int dt, uintptr_t st) {
+    launch_silu_f32(CP(in), ldi, P(out), ldo, T, n, dt, S(st));
+  });
+  m.def("delta_gates", [](uintptr_t a, uintptr_t b, int64_t ld, uintptr_t A_log, uintptr_t dtb, uintptr_t gates, int T,
+                          int H, int dt, uintptr_t st) {
+    launch_delta_gates(CP(a), CP(b), ld, CP(A_log), CP(dtb), P(gates), T, H, dt, S(st));
   });
   m.def("rope_bias_cache", [](uintptr_t proj, int64_t ldp, int off_q, int off_k, int off_v, uintptr_t bias,
                               uintptr_t pos, uintptr_t cs, int npos, int rot, uintptr_t qout, uintptr_t kc,

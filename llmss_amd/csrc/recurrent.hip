@@ -59,6 +59,7 @@ struct RecArgs {
   float* out;  // [T, H * vdim]
   int64_t ldo;
   int H, G, dim, vdim, silu_in;
+  int gates_ready;  // delta: a / b already hold g / beta (delta_gates_kernel), nothing left to compute while staging
 };
 
 // TQ: storage of q / k / v; TP: storage of a / b. R: state values per lane, P lanes per column. Staging: every
@@ -152,7 +153,8 @@ __global__ __launch_bounds__(256) void recurrence_kernel(RecArgs A, int P, int c
       }
       if (has_s) {
         float v = pre[jj * REC_NE + REC_NE - 1];
-        if (threadIdx.x == 0) {
+        if (A.gates_ready) {
+        } else if (threadIdx.x == 0) {
           v = 1.0f / (1.0f + expf(-v));
         } else {
           const float z = v + dtb;
@@ -268,12 +270,53 @@ static void recurrence_t(const RecArgs& A, int B, hipStream_t st) {
 void launch_recurrence(int mode, const void* q, const void* k, const void* v, int64_t ldq, int64_t ldk, int64_t ldv,
                        const void* ab, int64_t ldab, int off_a, int off_b, const void* decay, const void* dt_bias,
                        void* state, const void* cu, const void* ctx, const void* sslots, void* out, int64_t ldo, int B,
-                       int H, int G, int dim, int vdim, int silu_in, int dq, int dp, hipStream_t st) {
+                       int H, int G, int dim, int vdim, int silu_in, int gates_ready, int dq, int dp, hipStream_t st) {
   if (B == 0) return;
   if (G < 1 || H % G) throw std::runtime_error("recurrence: heads must be a multiple of the key heads");
   RecArgs A{q, k, v, ldq, ldk, ldv, ab, ldab, off_a, off_b, (const float*)decay, (const float*)dt_bias, (float*)state,
-            (const int*)cu, (const int*)ctx, (const int*)sslots, (float*)out, ldo, H, G, dim, vdim, silu_in};
+            (const int*)cu, (const int*)ctx, (const int*)sslots, (float*)out, ldo, H, G, dim, vdim, silu_in, gates_ready};
   if (mode == 0) DISPATCH_T(dq, TQ, (recurrence_t<TQ, float, 0>(A, B, st)));
   else DISPATCH_T(dq, TQ, DISPATCH_T(dp, TP, (recurrence_t<TQ, TP, 1>(A, B, st))));
+  HIP_CHECK_LAUNCH();
+}
+
+// Steps with long portions prepare what every workgroup of a head would otherwise recompute while staging:
+// out[t, c] = silu(in[t, c]) in fp32 (the decay recurrence's q | k | v), and the delta rule's per-token scalars
+// gates[t, h] = g = exp(-exp(A_log[h]) softplus(a[t, h] + dt_bias[h])), gates[t, H + h] = beta = sigmoid(b[t, h]).
+template <typename T>
+__global__ __launch_bounds__(256) void silu_f32_kernel(const T* __restrict__ in, int64_t ldi, float* __restrict__ out,
+                                                       int64_t ldo, int n) {
+  const int t = blockIdx.x;
+  for (int c = blockIdx.y * blockDim.x + threadIdx.x; c < n; c += gridDim.y * blockDim.x) {
+    const float v = El<T>::ld(in + (int64_t)t * ldi + c);
+    out[(int64_t)t * ldo + c] = v / (1.0f + (sizeof(T) == 2 ? __expf(-v) : expf(-v)));
+  }
+}
+
+void launch_silu_f32(const void* in, int64_t ldi, void* out, int64_t ldo, int T_, int n, int dt, hipStream_t st) {
+  if (T_ == 0 || n == 0) return;
+  dim3 g(T_, std::min(32, (n + 255) / 256));
+  DISPATCH_T(dt, T, (silu_f32_kernel<T><<<g, 256, 0, st>>>((const T*)in, ldi, (float*)out, ldo, n)));
+  HIP_CHECK_LAUNCH();
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void delta_gates_kernel(const T* __restrict__ a, const T* __restrict__ b, int64_t ld,
+                                                          const float* __restrict__ A_log,
+                                                          const float* __restrict__ dt_bias,
+                                                          float* __restrict__ gates, int T_, int H) {
+  const int e = blockIdx.x * blockDim.x + threadIdx.x;
+  if (e >= T_ * H) return;
+  const int t = e / H, h = e - t * H;
+  const float z = El<T>::ld(a + (int64_t)t * ld + h) + dt_bias[h];
+  gates[(int64_t)t * 2 * H + h] = expf(-expf(A_log[h]) * (z > 20.f ? z : log1pf(expf(z))));
+  gates[(int64_t)t * 2 * H + H + h] = 1.0f / (1.0f + expf(-El<T>::ld(b + (int64_t)t * ld + h)));
+}
+
+void launch_delta_gates(const void* a, const void* b, int64_t ld, const void* A_log, const void* dt_bias, void* gates,
+                        int T_, int H, int dt, hipStream_t st) {
+  if (T_ == 0) return;
+  DISPATCH_T(dt, T, (delta_gates_kernel<T><<<(T_ * H + 255) / 256, 256, 0, st>>>(
+      (const T*)a, (const T*)b, ld, (const float*)A_log, (const float*)dt_bias, (float*)gates, T_, H)));
   HIP_CHECK_LAUNCH();
 }

@@ -1196,11 +1196,20 @@ def decay_recurrence(q, k, v, decay, state, cu, ctx_lens, state_slots, heads, di
     T, B, out = _rec_common(q, k, v, state, cu, ctx_lens, state_slots, heads, heads, dim, vdim)
     _f32c(decay, "decay")
     _check(decay.numel() == heads, "decay [heads]")
+    if T and silu_in and T > B:
+        # portions: every workgroup of a head stages the head's whole q and k, so the activation is applied once
+        # beforehand (fp32 rows) instead of in each of them
+        nqk, nv = heads * dim, heads * vdim
+        act = torch.empty(T, 2 * nqk + nv, dtype=torch.float32, device=q.device)
+        for src, off, n in ((q, 0, nqk), (k, nqk, nqk), (v, 2 * nqk, nv)):
+            lib().silu_f32(src.data_ptr(), src.stride(0), act.data_ptr() + 4 * off, act.stride(0), T, n, _dt(src, "q"),
+                           _stream())
+        q, k, v, silu_in = act[:, :nqk], act[:, nqk:2 * nqk], act[:, 2 * nqk:], False
     if T:
         lib().recurrence(0, q.data_ptr(), k.data_ptr(), v.data_ptr(), q.stride(0), k.stride(0), v.stride(0), 0, 0, 0, 0,
                          decay.data_ptr(), 0, state.data_ptr(), cu.data_ptr(), ctx_lens.data_ptr(),
                          state_slots.data_ptr(), out.data_ptr(), heads * vdim, B, heads, heads, dim, vdim,
-                         int(bool(silu_in)), _dt(q, "q"), 0, _stream())
+                         int(bool(silu_in)), 0, _dt(q, "q"), 0, _stream())
     return out
 
 
@@ -1215,11 +1224,17 @@ def delta_recurrence(q, k, v, a, b_, A_log, dt_bias, state, cu, ctx_lens, state_
     _check(a.dtype == b_.dtype and a.stride(0) == b_.stride(0) and a.shape[0] == T and b_.shape[0] == T
            and a.untyped_storage().data_ptr() == b_.untyped_storage().data_ptr(), "a and b: columns of one tensor")
     off_b = (b_.data_ptr() - a.data_ptr()) // a.element_size()
+    ready = 0
+    if T > B:  # portions: the per-token decay and write strength once per (token, head), not per workgroup
+        gates = torch.empty(T, 2 * heads, dtype=torch.float32, device=q.device)
+        lib().delta_gates(a.data_ptr(), b_.data_ptr(), a.stride(0), A_log.data_ptr(), dt_bias.data_ptr(),
+                          gates.data_ptr(), T, heads, _dt(a, "a"), _stream())
+        a, off_b, ready = gates, heads, 1
     if T:
         lib().recurrence(1, q.data_ptr(), k.data_ptr(), v.data_ptr(), q.stride(0), k.stride(0), v.stride(0),
                          a.data_ptr(), a.stride(0), 0, int(off_b), A_log.data_ptr(), dt_bias.data_ptr(),
                          state.data_ptr(), cu.data_ptr(), ctx_lens.data_ptr(), state_slots.data_ptr(), out.data_ptr(),
-                         heads * vdim, B, heads, kv_heads, dim, vdim, 0, _dt(q, "q"), _dt(a, "a"), _stream())
+                         heads * vdim, B, heads, kv_heads, dim, vdim, 0, ready, _dt(q, "q"), _dt(a, "a"), _stream())
     return out
 
 
