@@ -4,7 +4,7 @@ blocks, rotary grouped-query attention, gated feed-forward) at equal size, rando
 
 "Equal size": same width, layer count, vocabulary and feed-forward width; the dense model's attention has the heads,
 key/value heads and head size of Babotar's attention branch. Babotar's layers follow the pattern parallel, parallel,
-decay, parallel (repeated), with two residual streams and a three-tap input convolution.
+decay, parallel (repeated), with two residual streams and a four-tap input convolution.
 """
 from __future__ import annotations
 
@@ -26,8 +26,8 @@ SIZES = {
 
 def babotar_dict(s, max_positions=8192):
     par = dict(type="parallel", mlp=dict(kind="dense", ff=s["ff"]), mixer=dict(
-        left=dict(heads=s["heads"], kv_heads=s["kv"], dim=s["dim"], vdim=s["dim"], scale=s["dim"] ** -0.5, softcap=50.0,
-                  rot=dict(base=10000.0, dims=s["rot"], scaling=dict(factor=4.0, original=2048, fast=32.0, slow=1.0))),
+        left=dict(heads=s["heads"], kv_heads=s["kv"], dim=s["dim"], vdim=s["dim"], scale=s["dim"] ** -0.5, softcap=30.0,
+                  rot=dict(base=10000.0, dims=s["rot"], scaling=dict(factor=4.0, original=4096, fast=16.0, slow=2.0))),
         right=dict(heads=s["dheads"], kv_heads=s["dkv"], dim=s["ddim"], vdim=s["dvdim"], conv=4),
         left_scale=1.0, right_scale=1.0))
     lig = dict(type="lightning", mlp=dict(kind="dense", ff=s["ff"]), mixer=dict(
@@ -35,7 +35,7 @@ def babotar_dict(s, max_positions=8192):
         decay=[1.0 - 2.0 ** (-3 - 5 * i / max(1, s["lheads"] - 1)) for i in range(s["lheads"])]))
     layers = [lig if i % 4 == 2 else par for i in range(s["layers"])]
     return dict(architecture="Babotar", vocab=s["vocab"], width=s["width"], max_positions=max_positions,
-                norm=dict(eps=1e-6), residual_mult=1.0, streams=2, canon=dict(taps=3), layers=layers)
+                norm=dict(eps=1e-6), residual_mult=1.0, streams=2, canon=dict(taps=4), layers=layers)
 
 
 def build(kind, s, dev):

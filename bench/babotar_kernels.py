@@ -108,15 +108,15 @@ def main():
         add("add_norm", phase, t, bytes_=T * W * 2 * 4, like="stream_add_norm")
         # ---- input convolution (no Llama counterpart)
         hf = rn(T, W, dt=torch.float32)
-        cw, tail = rn(W, 3), torch.zeros(B, 2, W, device=dev)
+        cw, tail = rn(W, 4), torch.zeros(B, 3, W, device=dev)
         t = timed(lambda: ops.causal_conv(hf, cw, tail, cu, cl, ss, True, False, bf))
-        add("causal_conv (3 taps, + tail)", phase, t, bytes_=T * W * (4 + 2))
+        add("causal_conv (4 taps, + tail)", phase, t, bytes_=T * W * (4 + 2))
         # ---- rotation + bias + cache write (Llama: rope_cache)
         nq, nk, nv = H * D, G * D, G * D
         proj = rn(T, nq + nk + nv)
         bias = rn(nq + nk + nv)
         kc, vc = rn(B * nblk, bs, nk), rn(B * nblk, bs, nv)
-        tab = ops.rope_angle_table(8192, rot, 10000.0, (4.0, 2048.0, 32.0, 1.0)).to(dev)
+        tab = ops.rope_angle_table(8192, rot, 10000.0, (4.0, 4096.0, 16.0, 2.0)).to(dev)
         t = timed(lambda: ops.rope_bias_cache(proj, 0, nq, nq + nk, bias, pos, tab, rot, kc, vc, slots, H, G, D, D))
         add("rope_bias_cache", phase, t, bytes_=T * ((nq + nk + nv) * 2 + nq * 4 + (nk + nv) * 2))
         # ---- attention
@@ -124,7 +124,7 @@ def main():
         talk = rn(H, H, dt=torch.float32)
         fl = pairs * H * 2 * (D + G * D)  # scores + weighted sums over all G value groups
         by = (T * nq * 4 + B * ctx * (nk + nv) * 2 + T * H * G * D * 4) if phase == "decode" else 0
-        f_attn = lambda: ops.sink_attn(qf, kc, vc, bt, cu, cl, H, G, D, D, D ** -0.5, 50.0, True, max_qlen=q)
+        f_attn = lambda: ops.sink_attn(qf, kc, vc, bt, cu, cl, H, G, D, D, D ** -0.5, 30.0, True, max_qlen=q)
         t = timed(f_attn, iters=3, warm=1)
         add("sink_attn (all value groups)", phase, t, flops=fl, bytes_=by)
         O = f_attn()

@@ -468,10 +468,10 @@ _PRESETS: Dict[str, Dict[str, Any]] = {
                                              kv_from=0),
                                   mlp=dict(kind="moe", router=dict(experts=4, top=1), expert=dict(ff=16, limit=2.0))),
                          ]),
-    # sequential per-layer design: two residual streams, input convolution, a parallel (attention | delta rule) layer,
+    # sequential per-layer design: three residual streams, input convolution, a parallel (attention | delta rule) layer,
     # a decay layer without a feed-forward, grouped heads and partial rotation
     "tiny-babotar": dict(architecture="Babotar", vocab=211, width=48, max_positions=256, norm=dict(eps=1e-5),
-                         residual_mult=0.5, streams=2, canon=dict(taps=3),
+                         residual_mult=0.5, streams=3, canon=dict(taps=2),
                          layers=[
                              dict(type="parallel",
                                   mixer=dict(left=dict(heads=4, kv_heads=2, dim=16, vdim=12, scale=0.2, softcap=30.0,

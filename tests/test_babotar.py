@@ -63,7 +63,7 @@ CONFIGS = {
     # one stream with learned weights, two-tap input convolution; head sizes the kernels tile (64, 128, above 128)
     "wide": dict(architecture="Babotar", vocab=83, width=64, max_positions=160, norm=dict(eps=1e-6),
                  residual_mult=1.5, streams=1, canon=dict(taps=2), layers=[
-        par(left(4, 2, 64, 128, 0.125, softcap=40.0, rot=dict(base=20000.0, dims=32, scaling=YARN)),
+        par(left(4, 2, 64, 128, 0.125, softcap=40.0, rot=dict(base=30000.0, dims=32, scaling=YARN)),
             dict(heads=2, kv_heads=1, dim=128, vdim=64, conv=4), 0.9, 0.9, ff=128),
         lig(2, 160, 72, [0.9, 0.999], ff=64),
     ]),
