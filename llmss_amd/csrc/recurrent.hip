@@ -69,14 +69,16 @@ struct RecArgs {
 template <typename TQ, typename TP, int R, int MODE>
 __global__ __launch_bounds__(256) void recurrence_kernel(RecArgs A, int P, int cols) {
   extern __shared__ __attribute__((aligned(16))) float sm[];
-  const int b = blockIdx.x, h = blockIdx.y;
+  // sequences in reverse step order, slowest in the grid: the step's long portions (they come last) are dispatched
+  // first, one per SIMD, and the single-token sequences fill in behind them
+  const int b = gridDim.z - 1 - blockIdx.z, h = blockIdx.x, zb = blockIdx.y;
   const int dim = A.dim, vdim = A.vdim;
   const int g = h / (A.H / A.G);
   const int qlen = A.cu[b + 1] - A.cu[b];
   if (qlen <= 0) return;
   const int t0 = A.cu[b], n = A.ctx[b], slot = A.sslots[b];
   const int cidx = min((int)threadIdx.x / P, cols - 1);
-  const int col = blockIdx.z * cols + cidx, part = threadIdx.x % P;
+  const int col = zb * cols + cidx, part = threadIdx.x % P;
   const bool live = col < vdim && (int)threadIdx.x < cols * P;
   if (slot < 0 || n <= 0) {
     if (live && part == 0)
@@ -124,7 +126,7 @@ __global__ __launch_bounds__(256) void recurrence_kernel(RecArgs A, int P, int c
       if (e - dimp < dim)
         has[k] = true, ld[k] = A.ldq, src[k] = (const TQ*)A.q + (int64_t)t0 * A.ldq + (int64_t)g * dim + (e - dimp);
     } else if (e < 2 * dimp + cols) {
-      const int c = blockIdx.z * cols + (e - 2 * dimp);
+      const int c = zb * cols + (e - 2 * dimp);
       if (c < vdim) has[k] = true, ld[k] = A.ldv, src[k] = (const TQ*)A.v + (int64_t)t0 * A.ldv + (int64_t)h * vdim + c;
     }
   }
@@ -259,8 +261,8 @@ static void recurrence_t(const RecArgs& A, int B, hipStream_t st) {
   const int per = (2 * dimp + cols + 2 + 3) & ~3;
   const int threads = ((std::max(cols * P, (2 * dimp + cols + REC_NE - 2) / (REC_NE - 1)) + 63) / 64) * 64;
   if (threads > 256) throw std::runtime_error("recurrence: too many numbers per token to stage");
-  dim3 g(B, A.H, (vdim + cols - 1) / cols);
-  if (A.H > 65535 || g.z > 65535) throw std::runtime_error("recurrence: too many heads or columns");
+  dim3 g(A.H, (vdim + cols - 1) / cols, B);
+  if (B > 65535 || g.y > 65535) throw std::runtime_error("recurrence: too many sequences or columns");
   const size_t lds = ((size_t)REC_CT * per + 4 * 128) * 4;  // + room for the last token's reads past its k / q
   if (R == 32) recurrence_kernel<TQ, TP, 32, MODE><<<g, threads, lds, st>>>(A, P, cols);
   else if (R == 64) recurrence_kernel<TQ, TP, 64, MODE><<<g, threads, lds, st>>>(A, P, cols);

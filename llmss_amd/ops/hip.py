@@ -1274,8 +1274,8 @@ def rope_bias_cache(proj, off_q, off_k, off_v, bias, positions, table, rot, k_ca
 def sink_attn(q, k_cache, v_cache, block_tables, cu, ctx_lens, heads, kv_heads, dim, vdim, scale, softcap,
               all_groups, max_qlen=0, num_decode=0):
     """``max_qlen`` (the longest portion of the step, known on the host) > 0: a bf16 cache of a shape the matrix-core
-    kernel is built for runs on it, portions and single rows alike (``num_decode`` leading single-row sequences are
-    part of its grid); everything else runs the vector kernel."""
+    kernel is built for runs on it, the ``num_decode`` leading single-row sequences in one launch and the portions
+    in another; everything else runs the vector kernel."""
     T = q.shape[0]
     _rows(q, "q", heads * dim, torch.float32)
     _check(q.is_contiguous(), "q contiguous")
@@ -1295,9 +1295,14 @@ def sink_attn(q, k_cache, v_cache, block_tables, cu, ctx_lens, heads, kv_heads, 
             and k_cache.data_ptr() % 16 == 0 and v_cache.data_ptr() % 16 == 0 and os.environ.get("LLMSS_SINK_MFMA", "1") != "0")
     common = (heads, kv_heads, dim, vdim, k_cache.shape[1], float(scale), float(softcap or 0.0), int(bool(all_groups)))
     if mfma:
-        lib().sink_attn_mfma(q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), block_tables.data_ptr(),
-                             block_tables.shape[1], cu.data_ptr(), ctx_lens.data_ptr(), out.data_ptr(), B,
-                             int(max_qlen), *common, _stream())
+        # the leading single-row sequences get a grid of their own (one row block each): in the portions' grid every
+        # one of them would launch a whole prompt's worth of workgroups that exit at once, and those are not free
+        maxb = block_tables.shape[1]
+        for first, n, ql in ((0, nd, 1), (nd, B - nd, int(max_qlen))):
+            if n > 0:
+                lib().sink_attn_mfma(q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
+                                     block_tables.data_ptr() + 4 * first * maxb, maxb, cu.data_ptr() + 4 * first,
+                                     ctx_lens.data_ptr() + 4 * first, out.data_ptr(), n, ql, *common, _stream())
     else:
         lib().sink_attn(q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), block_tables.data_ptr(),
                         block_tables.shape[1], cu.data_ptr(), ctx_lens.data_ptr(), out.data_ptr(), T, B, *common,
