@@ -520,6 +520,26 @@ __global__ __launch_bounds__(256) void talk_mix_kernel(const float* __restrict__
   const int rep = H / G;
   const int RVtot = talk ? G * vdim : vdim;
   const float* Ot = O + (int64_t)t * H * RVtot;
+  if ((vdim & 3) == 0) {  // four columns per thread, 16-byte reads
+    for (int e = threadIdx.x * 4; e < H * vdim; e += blockDim.x * 4) {
+      const int h = e / vdim, v = e % vdim;
+      f32x4 a;
+      if (talk) {
+        a = f32x4{0.f, 0.f, 0.f, 0.f};
+        const int col = (h / rep) * vdim + v;
+        for (int hh = 0; hh < H; ++hh) {
+          const float w = talk[h * H + hh];
+          const f32x4 x = *reinterpret_cast<const f32x4*>(Ot + (int64_t)hh * RVtot + col);
+          a[0] = fmaf(w, x[0], a[0]), a[1] = fmaf(w, x[1], a[1]), a[2] = fmaf(w, x[2], a[2]), a[3] = fmaf(w, x[3], a[3]);
+        }
+      } else {
+        a = *reinterpret_cast<const f32x4*>(Ot + (int64_t)h * RVtot + v);
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i) El<T>::st(y + (int64_t)t * ldy + e + i, a[i] * c);
+    }
+    return;
+  }
   for (int e = threadIdx.x; e < H * vdim; e += blockDim.x) {
     const int h = e / vdim, v = e % vdim;
     float a;

@@ -1238,12 +1238,6 @@ def delta_recurrence(q, k, v, a, b_, A_log, dt_bias, state, cu, ctx_lens, state_
     return out
 
 
-def rope_angle_table(npos, dims, base, scaling=None):
-    from . import reference as ref
-
-    return ref.rope_angle_table(npos, dims, base, scaling)
-
-
 def rope_bias_cache(proj, off_q, off_k, off_v, bias, positions, table, rot, k_cache, v_cache, slots, heads, kv_heads,
                     dim, vdim):
     T = proj.shape[0]
@@ -1271,6 +1265,9 @@ def rope_bias_cache(proj, off_q, off_k, off_v, bias, positions, table, rot, k_ca
     return q
 
 
+_SINK_MFMA = os.environ.get("LLMSS_SINK_MFMA", "1") != "0"  # 0: every shape on the vector kernel (A/B runs)
+
+
 def sink_attn(q, k_cache, v_cache, block_tables, cu, ctx_lens, heads, kv_heads, dim, vdim, scale, softcap,
               all_groups, max_qlen=0, num_decode=0):
     """``max_qlen`` (the longest portion of the step, known on the host) > 0: a bf16 cache of a shape the matrix-core
@@ -1292,7 +1289,7 @@ def sink_attn(q, k_cache, v_cache, block_tables, cu, ctx_lens, heads, kv_heads, 
     nd = int(num_decode)
     _check(0 <= nd <= B, "num_decode outside the step")
     mfma = (k_cache.dtype == torch.bfloat16 and max_qlen > 0 and lib().sink_attn_mfma_ok(dim, vdim)
-            and k_cache.data_ptr() % 16 == 0 and v_cache.data_ptr() % 16 == 0 and os.environ.get("LLMSS_SINK_MFMA", "1") != "0")
+            and k_cache.data_ptr() % 16 == 0 and v_cache.data_ptr() % 16 == 0 and _SINK_MFMA)
     common = (heads, kv_heads, dim, vdim, k_cache.shape[1], float(scale), float(softcap or 0.0), int(bool(all_groups)))
     if mfma:
         # the leading single-row sequences get a grid of their own (one row block each): in the portions' grid every
