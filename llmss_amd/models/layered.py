@@ -17,7 +17,7 @@ beside them. Besides pages of the shared pool a mixer may own per-sequence state
 inputs of a convolution): ``LayerCache.state`` tensors indexed by the scheduler's state slot of each sequence
 (``StepInput.state_slots``); a portion that starts at position 0 starts from an empty state.
 
-Mixer ``parallel`` (ops: linear_f, rope_bias_cache, sink_attn, talk_mix, causal_conv, delta_recurrence,
+Mixer ``parallel`` (ops: linear_f, rope_bias_cache, sink_attn_mix = sink_attn + talk_mix, causal_conv, delta_recurrence,
 gated_group_norm): softmax attention with a sink, soft cap, partial scaled rotation and head mixing beside a gated
 delta rule, one input GEMM and one output GEMM for both. Mixer ``lightning`` (decay_recurrence, gated_group_norm):
 linear attention with a constant decay per head. Feed-forward ``dense`` (glu_act): gated, tanh-form GELU.
@@ -132,12 +132,12 @@ class ParallelMixer:
                                 a.rot.dims if a.rot is not None else 0, kc, vc, inp.slots, a.heads, a.kv_heads, a.dim,
                                 a.vdim)
         single = inp.kind == "decode"
-        O = ops.sink_attn(q, kc, vc, inp.block_tables, cu, inp.ctx_lens, a.heads, a.kv_heads, a.dim, a.vdim, a.scale,
-                          a.softcap, W.talk is not None, max_qlen=1 if single else max(1, inp.max_seqlen),
-                          num_decode=0 if single else inp.num_decode)
         nl, nr = a.heads * a.vdim, r.heads * r.vdim
         both = torch.empty(T, nl + nr, dtype=dt, device=h.device)  # [left | right] rows for the one output GEMM
-        ops.talk_mix(O, W.talk, spec.left_scale, a.heads, a.kv_heads, a.vdim, out=both[:, :nl])
+        ops.sink_attn_mix(q, kc, vc, inp.block_tables, cu, inp.ctx_lens, W.talk, spec.left_scale, a.heads, a.kv_heads,
+                          a.dim, a.vdim, a.scale, a.softcap, both[:, :nl],
+                          max_qlen=1 if single else max(1, inp.max_seqlen), num_decode=0 if single else inp.num_decode,
+                          max_ctx=inp.max_ctx)
         # right: short convolution + SiLU on q | k | v, then the gated delta rule over the sequence's matrix state
         nqk = r.kv_heads * r.dim
         qkv = ops.causal_conv(proj[:, c["rq"]:c["rq"] + 2 * nqk + nr], W.conv, st["tail"], cu, inp.ctx_lens,

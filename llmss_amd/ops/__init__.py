@@ -185,5 +185,6 @@ decay_recurrence = _route("decay_recurrence")
 delta_recurrence = _route("delta_recurrence")
 rope_bias_cache = _route("rope_bias_cache")
 sink_attn = _route("sink_attn")
+sink_attn_mix = _route("sink_attn_mix")
 talk_mix = _route("talk_mix")
 rope_angle_table = ref.rope_angle_table

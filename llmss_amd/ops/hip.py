@@ -1307,6 +1307,18 @@ def sink_attn(q, k_cache, v_cache, block_tables, cu, ctx_lens, heads, kv_heads, 
     return out
 
 
+def sink_attn_mix(q, k_cache, v_cache, block_tables, cu, ctx_lens, talk, c, heads, kv_heads, dim, vdim, scale, softcap,
+                  out, max_qlen=0, num_decode=0, max_ctx=0):
+    """Sink attention, head mixing and the branch scale, written to ``out`` [T, heads * vdim]: sink_attn (weighted
+    sums of every head over all value groups when ``talk`` is given) followed by talk_mix. (A two-pass form for steps
+    of single rows - scores of every head first, then mixed weights against each head's own group, so that keys and
+    values are each read once - was measured at twice the time of the matrix-core kernel at 64 rows x 1024 keys:
+    too few workgroups without a split over keys. It is not kept.)"""
+    O = sink_attn(q, k_cache, v_cache, block_tables, cu, ctx_lens, heads, kv_heads, dim, vdim, scale, softcap,
+                  talk is not None, max_qlen=max_qlen, num_decode=num_decode)
+    return talk_mix(O, talk, c, heads, kv_heads, vdim, out=out)
+
+
 def talk_mix(O, talk, c, heads, kv_heads, vdim, out=None, out_dtype=None):
     T = O.shape[0]
     R = kv_heads * vdim if talk is not None else vdim

@@ -791,6 +791,17 @@ def sink_attn(q, k_cache, v_cache, block_tables, cu, ctx_lens, heads: int, kv_he
     return out
 
 
+def sink_attn_mix(q, k_cache, v_cache, block_tables, cu, ctx_lens, talk, c: float, heads: int, kv_heads: int, dim: int,
+                  vdim: int, scale: float, softcap: float, out, max_qlen: int = 0, num_decode: int = 0,
+                  max_ctx: int = 0):
+    """Sink attention, head mixing (``talk`` [heads, heads] or None) and the scale ``c`` in one op, written to
+    ``out`` [T, heads * vdim]. ``max_qlen``, ``num_decode`` and ``max_ctx`` (an upper bound of every context length)
+    only steer the choice of GPU kernels."""
+    O = sink_attn(q, k_cache, v_cache, block_tables, cu, ctx_lens, heads, kv_heads, dim, vdim, scale, softcap,
+                  talk is not None)
+    return talk_mix(O, talk, c, heads, kv_heads, vdim, out=out)
+
+
 def talk_mix(O, talk, c: float, heads: int, kv_heads: int, vdim: int, out=None, out_dtype=None):
     """y[t, h, :] = c * sum_h' talk[h, h'] O[t, h', group(h) part] (talk None: c * O). [T, heads * vdim]."""
     T = O.shape[0]

@@ -350,3 +350,34 @@ def test_the_sink_takes_the_weight_when_every_score_is_low_and_the_cap_holds_hig
                                       10.0, None)
     close(O.reshape(20, -1), want.reshape(20, -1), dtype, "capped scores")
     assert torch.isfinite(O).all()
+
+
+@pytest.mark.parametrize("device,dtype", RUNS)
+@pytest.mark.parametrize("H,G,d,dv", [(4, 2, 16, 12), (8, 1, 8, 40), (6, 2, 64, 72), (3, 3, 24, 8), (16, 4, 128, 128),
+                                      (5, 1, 8, 8), (16, 2, 32, 300)])
+def test_a_step_of_single_rows_mixes_heads_before_it_meets_the_values(device, dtype, H, G, d, dv):
+    """Decoded rows only, one per sequence, contexts of unequal length (one of a single token): attention, head
+    mixing and the scale in one op, written into a view of a wider buffer."""
+    lens = [70, 33, 1, 129]
+    pg = Paged(lens, G, d, dv, 16, device, dtype, seed=3)
+    data = []
+    for i, n in enumerate(lens):
+        q, k, v = rnd(n, H, d, seed=50 + 3 * i), rnd(n, G, d, seed=51 + 3 * i, dtype=dtype), \
+            rnd(n, G, dv, seed=52 + 3 * i, dtype=dtype)
+        k[n // 2] *= 3.0  # one key stands out in the middle of each context
+        sl = torch.tensor(pg.slots(i, 0, n), device=device)
+        pg.kc.view(-1, G * d)[sl] = k.reshape(n, -1).to(dtype).to(device)
+        pg.vc.view(-1, G * dv)[sl] = v.reshape(n, -1).to(dtype).to(device)
+        data.append((q, k, v))
+    tk = torch.eye(H).double() * 0.5 + 0.4 * rnd(H, H, seed=9)
+    B = len(lens)
+    q = torch.stack([data[i][0][-1] for i in range(B)]).reshape(B, H * d).float().to(device)
+    out = torch.zeros(B, H * dv + 5, dtype=dtype, device=device)  # a view into a wider buffer, as the mixer passes
+    ops.sink_attn_mix(q, pg.kc, pg.vc, pg.bt(list(range(B)), device), i32(list(range(B + 1)), device), i32(lens, device),
+                      tk.float().to(device).contiguous(), 0.8, H, G, d, dv, d ** -0.5, 20.0, out[:, :H * dv],
+                      max_qlen=1, num_decode=0, max_ctx=pg.maxb * 16)
+    for i, n in enumerate(lens):
+        qq, k, v = data[i]
+        want = 0.8 * oracle.sink_talk_attention(qq, k, v, d ** -0.5, 20.0, tk)[-1].reshape(-1)
+        close(out[i, :H * dv], want, dtype, f"sequence {i}", scale=float(v.abs().max()))
+    assert float(out[:, H * dv:].float().abs().max()) == 0.0
