@@ -138,6 +138,9 @@ void launch_sink_attn(const void* q, const void* kc, const void* vc, const void*
                       const void* ctx, void* out, int T_, int B, int H, int G, int dim, int vdim, int bs, float scale,
                       float cap, int all, int dt, hipStream_t st);
 bool sink_attn_mfma_ok(int dim, int vdim);
+void launch_sink_attn_mfma(const void* q, const void* kc, const void* vc, const void* bt, int maxb, const void* cu,
+                           const void* ctx, void* out, int B, int max_qlen, int H, int G, int dim, int vdim, int bs,
+                           float scale, float cap, int all, hipStream_t st);
 void launch_talk_mix(const void* O, const void* talk, float c, void* y, int64_t ldy, int T_, int H, int G, int vdim,
                      int dt, hipStream_t st);
 
